@@ -1,0 +1,129 @@
+"""Helpers shared by the oracle tests (CPU) and the parity tests (GPU).
+
+`run_case(be, case)` replays one golden case -- the literal inputs of one of the reference's own
+operator tests -- through a backend `be` that offers the operator methods of `oracle.Oracle`
+(the HIP front-end offers the same ones) and returns the tensors the reference test exports.
+"""
+import numpy as np
+
+# north_star tolerance for fp32 results: 1e-4 relative / 1e-5 absolute
+RTOL, ATOL = 1e-4, 1e-5
+
+
+def get(case, key, kind="inputs"):
+    a = case[kind][key]
+    return np.array(a["data"], dtype=np.float64).reshape(a["shape"])
+
+
+def same_pad(n_in, k, s):
+    p = k - s if n_in % s == 0 else k - (n_in % s)
+    return max(p, 0), -(-n_in // s)
+
+
+def mse_dy(be, y, y_hat):
+    """Gradient of the reference tests' `reshape -> mse` wrapper w.r.t. y_hat
+    (reference: src/cpu/kernels.cu:110-113)."""
+    return be.mse_grad(y.reshape(y.shape[0], -1), y_hat.reshape(y.shape[0], -1)).reshape(y_hat.shape)
+
+
+def run_case(be, case):
+    op, p = case["op"], case["params"]
+    I = lambda k: get(case, k).astype(np.float32)
+    if op == "conv2d":
+        return {"y": be.conv2d(I("x"), I("k"), p["strides"])}
+    if op == "conv2d_grad":
+        x, k, y = I("x"), I("k"), I("y")
+        s = p["strides"]
+        pads = (same_pad(x.shape[1], k.shape[0], s[0])[0], same_pad(x.shape[2], k.shape[1], s[1])[0])
+        y_hat = be.conv2d(x, k, s)
+        dy = mse_dy(be, y, y_hat)
+        return {"y_hat": y_hat, "dy_hat": dy,
+                "dx": be.conv2d_input_grad(dy, k, s[0], x.shape[1:3]),
+                "dk": be.conv2d_kernel_grad(dy, x, s[0], pads, k.shape[:2]),
+                "loss": be.mse(y.reshape(y.shape[0], -1), y_hat.reshape(y.shape[0], -1))}
+    if op == "conv2d_transpose":
+        return {"y": be.conv2d_transpose(I("x"), I("k"), p["out_size"][1:3], p["strides"][0])}
+    if op == "conv2d_transpose_grad":
+        x, k, y = I("x"), I("k"), I("y")
+        s = p["strides"][0]
+        y_hat = be.conv2d_transpose(x, k, p["out_size"][1:3], s)
+        dy = mse_dy(be, y, y_hat)
+        return {"y_hat": y_hat, "dy_hat": dy,
+                "dx": be.conv2d_transpose_input_grad(dy, k, s, x.shape[1:3]),
+                "dk": be.conv2d_transpose_kernel_grad(dy, x, s, k.shape[:2]),
+                "loss": be.mse(y.reshape(y.shape[0], -1), y_hat.reshape(y.shape[0], -1))}
+    if op == "bias_add":
+        return {"out": be.bias_add(I("z"), I("b"))}
+    if op == "bias_add_grad":
+        z, b, y = I("z"), I("b"), I("y")
+        dy = mse_dy(be, y, be.bias_add(z, b))
+        return {"dy_hat": dy, "dx": dy, "db": be.bias_grad(dy)}
+    if op == "mat_sum_cols":
+        return {"out": be.bias_grad(I("x"))}
+    if op == "relu_leaky":
+        return {"out": be.relu_leaky(I("x"), p["alpha"])}
+    if op in ("relu", "tanh", "sigmoid"):
+        return {"out": getattr(be, op)(I("x"))}
+    if op in ("leaky_relu_grad", "relu_grad", "tanh_grad", "sigmoid_grad"):
+        x, y = I("x"), I("y")
+        fwd = {"leaky_relu_grad": lambda v: be.relu_leaky(v, p["alpha"]), "relu_grad": be.relu,
+               "tanh_grad": be.tanh, "sigmoid_grad": be.sigmoid}[op]
+        y_hat = fwd(x)
+        dy = mse_dy(be, y, y_hat)
+        if op == "leaky_relu_grad":
+            dx = be.leaky_relu_grad(x, dy, p["alpha"])
+        elif op == "relu_grad":
+            dx = be.relu_grad(x, dy)
+        else:  # tanh / sigmoid gradients take the forward OUTPUT
+            dx = getattr(be, op)(y_hat, dy)
+        return {"y_hat": y_hat, "dy_hat": dy, "dx": dx}
+    if op == "add":
+        return {"out": be.add(I("a"), I("b"))}
+    if op == "argmax_acc":
+        return {"acc": np.array(float(be.argmax_acc(I("y"), I("y_hat"))))}
+    if op == "sigmoid_cross_entropy":
+        x, y = I("x"), I("y")
+        return {"loss": np.array(be.sigmoid_cross_entropy(y.reshape(-1), x.reshape(-1))),
+                "dx": be.sigmoid_cross_entropy_grad(y, x)}
+    if op == "moment_update":
+        return {"out": be.moment_update(I("var"), I("dv"), p["c1"], p["c2"])}
+    if op == "moment_update2":
+        return {"out": be.moment_update2(I("var"), I("dv"), p["c1"], p["c2"])}
+    if op == "adam_update":
+        t, lrt = be.adam_lrt(p["t_before"], p["lr"], p["beta1"], p["beta2"])
+        assert t == 1.0
+        return {"out": be.adam_apply(I("x"), I("m"), I("v"), lrt, p["eps"])}
+    if op == "mat_mul_add":
+        return {"out": be.mat_mul_add(I("x"), I("w"), I("b"))}
+    if op in ("mm_mul", "tmm_mul", "mtm_mul"):
+        return {"out": getattr(be, op)(I("a"), I("b"))}
+    raise KeyError(op)
+
+
+def check_case(be, case, rtol=RTOL, atol=ATOL):
+    got = run_case(be, case)
+    for key, exp in case["expected"].items():
+        e = np.array(exp["data"], dtype=np.float64).reshape(exp["shape"])
+        g = np.asarray(got[key], dtype=np.float64).reshape(e.shape)
+        np.testing.assert_allclose(g, e, rtol=rtol, atol=atol,
+                                   err_msg="%s / %s (%s)" % (case["name"], key, case["source"]))
+
+
+GOLDEN_NAMES = [
+    "conv2d", "conv2d_padding", "conv2d_grad", "conv2d_padding_grad", "conv2d_transpose",
+    "conv2d_transpose_grad", "conv2d_bias_add", "conv2d_bias_add_grad", "vect_relu_leaky",
+    "vect_relu", "vect_tanh", "sigmoid", "leaky_relu_grad", "relu_grad", "tanh_grad",
+    "sigmoid_grad", "add", "argmax_accuracy", "sigmoid_cross_entropy", "moment_update",
+    "moment_update2", "adam_update", "mat_mul_add", "mat_mat_mul", "tmat_mat_mul",
+    "mat_tmat_mul", "mat_rvect_add", "mat_sum_cols"]
+
+
+def rand_conv_inputs(seed, N, H, W, C, kh, kw, O, s):
+    """Seeded inputs in the distributions the benchmark configurations name:
+    x ~ U(-1,1), k ~ N(0, 0.02), dy ~ U(-1,1)."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-1, 1, (N, H, W, C)).astype(np.float32)
+    k = (rng.standard_normal((kh, kw, C, O)) * 0.02).astype(np.float32)
+    Ho, Wo = -(-H // s), -(-W // s)
+    dy = rng.uniform(-1, 1, (N, Ho, Wo, O)).astype(np.float32)
+    return x, k, dy
