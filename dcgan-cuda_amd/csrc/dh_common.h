@@ -1,0 +1,76 @@
+// Internal helpers shared by the HIP translation units of libdcgan_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "dcgan_hip.h"
+
+namespace dh
+{
+
+// Records `msg` as the calling thread's last error and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail_hip(hipError_t err, const char* what);
+// Makes sure a device is selected and the library state exists (device 0 by default).
+int ensure_init();
+// Scratch arena of the current device, at least `bytes` large (grows, never shrinks).
+int workspace(size_t bytes, void** ptr);
+int num_cus();
+
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+#define DH_TRY(expr)                                   \
+    do {                                               \
+        int dh_rc_ = (expr);                           \
+        if (dh_rc_ != 0) return dh_rc_;                \
+    } while (0)
+
+#define DH_HIP(expr)                                                \
+    do {                                                            \
+        hipError_t dh_e_ = (expr);                                  \
+        if (dh_e_ != hipSuccess) return ::dh::fail_hip(dh_e_, #expr); \
+    } while (0)
+
+// Call right after a kernel launch: reports launch-configuration errors.
+#define DH_LAUNCH_CHECK(name)                                              \
+    do {                                                                   \
+        hipError_t dh_e_ = hipGetLastError();                              \
+        if (dh_e_ != hipSuccess) return ::dh::fail_hip(dh_e_, name);       \
+    } while (0)
+
+// Division of a non-negative 31-bit integer by a runtime constant without the hardware's
+// ~40-instruction integer divide (Granlund-Montgomery round-up method):
+//   q = (umulhi(n, mul) + n) >> shift   for 0 <= n < 2^31, 1 <= d < 2^31.
+struct FastDiv
+{
+    uint32_t mul;
+    uint32_t shift;
+    uint32_t d;
+
+    FastDiv() : mul(0), shift(0), d(1) {}
+    explicit FastDiv(uint32_t div) : d(div ? div : 1)
+    {
+        uint32_t l = 0;
+        while ((1ull << l) < d) ++l;
+        shift = l;
+        mul = (uint32_t)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    }
+    __host__ __device__ inline uint32_t div(uint32_t n) const
+    {
+#if defined(__HIP_DEVICE_COMPILE__)
+        return (__umulhi(n, mul) + n) >> shift;
+#else
+        return (uint32_t)((((uint64_t)n * mul) >> 32) + n) >> shift;
+#endif
+    }
+    __host__ __device__ inline void divmod(uint32_t n, uint32_t& q, uint32_t& r) const
+    {
+        q = div(n);
+        r = n - q * d;
+    }
+};
+
+}  // namespace dh

@@ -1,0 +1,608 @@
+// HBM-bound operators of the hot path: bias add / bias gradient, activations and their
+// gradients, tensor add, the Adam kernels and the small loss reductions.
+// Every kernel streams its operands once with 16-byte accesses where the sizes allow and has a
+// scalar tail, so any length and any alignment is accepted.
+//
+// Reference counterparts: src/gpu/relu.cu, src/gpu/sigmoid.cu, src/gpu/sum.cu, src/gpu/update.cu,
+// mvrow_add in src/gpu/matmul.cu; arithmetic as in src/cpu/ops.hxx.
+#include "dh_common.h"
+
+using namespace dh;
+
+namespace
+{
+
+constexpr int TPB = 256;
+
+inline bool aligned16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
+
+inline unsigned grid_for(size_t work, int per_cu = 8)
+{
+    size_t blocks = (work + TPB - 1) / TPB;
+    const size_t cap = (size_t)num_cus() * per_cu;
+    if (blocks > cap) blocks = cap;
+    return blocks == 0 ? 1u : (unsigned)blocks;
+}
+
+// ---- generic element-wise maps ----------------------------------------------------------------
+
+struct OpRelu { __device__ float operator()(float x) const { return x < 0.f ? 0.f : x; } };
+struct OpLeaky { float alpha; __device__ float operator()(float x) const { return x < 0.f ? alpha * x : x; } };
+struct OpTanh { __device__ float operator()(float x) const { return tanhf(x); } };
+struct OpSigmoid { __device__ float operator()(float x) const { return 1.f / (1.f + expf(-x)); } };
+
+struct OpReluGrad { __device__ float operator()(float z, float d) const { return z > 0.f ? d : 0.f; } };
+struct OpLeakyGrad { float alpha; __device__ float operator()(float z, float d) const { return z < 0.f ? alpha * d : d; } };
+struct OpTanhGrad { __device__ float operator()(float t, float d) const { return (1.f - t * t) * d; } };
+struct OpSigmoidGrad { __device__ float operator()(float s, float d) const { return s * (1.f - s) * d; } };
+struct OpAdd { __device__ float operator()(float a, float b) const { return a + b; } };
+struct OpSceGrad { float inv_n; __device__ float operator()(float y, float x) const { return (1.f / (1.f + expf(-x)) - y) * inv_n; } };
+struct OpMseGrad { float coeff; __device__ float operator()(float y, float yh) const { return coeff * (yh - y); } };
+struct OpMoment { float a, b; __device__ float operator()(float m, float g) const { return a * m + b * g; } };
+struct OpMoment2 { float a, b; __device__ float operator()(float v, float g) const { return a * v + b * g * g; } };
+
+template <class F>
+__global__ __launch_bounds__(TPB) void map1(const float* __restrict__ x, float* __restrict__ out, size_t n, bool vec, F f)
+{
+    const size_t stride = (size_t)gridDim.x * TPB;
+    const size_t tid = (size_t)blockIdx.x * TPB + threadIdx.x;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride)
+        {
+            float4 v = reinterpret_cast<const float4*>(x)[i];
+            v.x = f(v.x); v.y = f(v.y); v.z = f(v.z); v.w = f(v.w);
+            reinterpret_cast<float4*>(out)[i] = v;
+        }
+        done = n4 * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride)
+        out[i] = f(x[i]);
+}
+
+// out may alias a (in-place moment updates) -- no __restrict__ on those two.
+template <class F>
+__global__ __launch_bounds__(TPB) void map2(const float* a, const float* __restrict__ b, float* out, size_t n, bool vec, F f)
+{
+    const size_t stride = (size_t)gridDim.x * TPB;
+    const size_t tid = (size_t)blockIdx.x * TPB + threadIdx.x;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride)
+        {
+            const float4 u = reinterpret_cast<const float4*>(a)[i];
+            const float4 w = reinterpret_cast<const float4*>(b)[i];
+            float4 v;
+            v.x = f(u.x, w.x); v.y = f(u.y, w.y); v.z = f(u.z, w.z); v.w = f(u.w, w.w);
+            reinterpret_cast<float4*>(out)[i] = v;
+        }
+        done = n4 * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride)
+        out[i] = f(a[i], b[i]);
+}
+
+template <class F>
+int run_map1(const char* who, const float* x, float* out, size_t n, void* stream, F f)
+{
+    DH_TRY(ensure_init());
+    if (n == 0) return 0;
+    if (!x || !out) return fail(DH_EINVAL, "%s: null tensor", who);
+    const bool vec = aligned16(x) && aligned16(out);
+    hipLaunchKernelGGL(map1<F>, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), x, out, n, vec, f);
+    DH_LAUNCH_CHECK(who);
+    return 0;
+}
+
+template <class F>
+int run_map2(const char* who, const float* a, const float* b, float* out, size_t n, void* stream, F f)
+{
+    DH_TRY(ensure_init());
+    if (n == 0) return 0;
+    if (!a || !b || !out) return fail(DH_EINVAL, "%s: null tensor", who);
+    const bool vec = aligned16(a) && aligned16(b) && aligned16(out);
+    hipLaunchKernelGGL(map2<F>, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), a, b, out, n, vec, f);
+    DH_LAUNCH_CHECK(who);
+    return 0;
+}
+
+__global__ __launch_bounds__(TPB) void fill_zero(float* __restrict__ out, size_t n, bool vec)
+{
+    const size_t stride = (size_t)gridDim.x * TPB;
+    const size_t tid = (size_t)blockIdx.x * TPB + threadIdx.x;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride)
+            reinterpret_cast<float4*>(out)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        done = n4 * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride)
+        out[i] = 0.f;
+}
+
+// ---- bias add: out[r,c] = z[r,c] + b[c] ---------------------------------------------------------
+// The flat index runs over the whole matrix; the column of a 4-chunk is (4*i) % cols.
+template <bool VEC>
+__global__ __launch_bounds__(TPB) void bias_add_kernel(const float* __restrict__ z, const float* __restrict__ b,
+                                                       float* __restrict__ out, size_t n, FastDiv fd_cols)
+{
+    const size_t stride = (size_t)gridDim.x * TPB;
+    const size_t tid = (size_t)blockIdx.x * TPB + threadIdx.x;
+    const uint32_t cols = fd_cols.d;
+    if (VEC)
+    {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride)
+        {
+            const uint32_t e = (uint32_t)(i * 4);
+            const uint32_t c = e - fd_cols.div(e) * cols;
+            float4 v = reinterpret_cast<const float4*>(z)[i];
+            const float4 w = *reinterpret_cast<const float4*>(b + c);
+            v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+            reinterpret_cast<float4*>(out)[i] = v;
+        }
+    }
+    else
+    {
+        for (size_t i = tid; i < n; i += stride)
+        {
+            const uint32_t e = (uint32_t)i;
+            out[i] = z[i] + b[e - fd_cols.div(e) * cols];
+        }
+    }
+}
+
+// ---- column sums (bias gradient), optionally fused with the activation gradient ------------------
+// Stage 1: the rows are cut into `chunks` contiguous ranges; a workgroup owns one range and one
+// tile of 256 columns.  For narrow matrices (cols <= 256) G = 256/cols consecutive rows are laid
+// side by side so that consecutive lanes still read consecutive addresses.  Each lane adds its
+// column serially; lanes of the same column are then added in lane order.  Stage 2 adds the
+// per-range sums in range order.  The result is therefore independent of scheduling.
+struct ActGrad
+{
+    int act;
+    float alpha;
+    __device__ float operator()(float ref, float d) const
+    {
+        switch (act)
+        {
+        case DH_ACT_RELU: return ref > 0.f ? d : 0.f;
+        case DH_ACT_LEAKY: return ref < 0.f ? alpha * d : d;
+        case DH_ACT_TANH: return (1.f - ref * ref) * d;
+        case DH_ACT_SIGMOID: return ref * (1.f - ref) * d;
+        default: return d;
+        }
+    }
+};
+
+template <bool FUSED>
+__global__ __launch_bounds__(TPB) void colsum_stage1(const float* __restrict__ a, const float* __restrict__ act_ref,
+                                                     float* __restrict__ dz, float* __restrict__ partial,
+                                                     size_t rows, uint32_t cols, uint32_t G, size_t rows_per_chunk,
+                                                     ActGrad g)
+{
+    __shared__ float lds[TPB];
+    const uint32_t t = threadIdx.x;
+    const size_t r_begin = (size_t)blockIdx.y * rows_per_chunk;
+    size_t r_end = r_begin + rows_per_chunk;
+    if (r_end > rows) r_end = rows;
+    float acc = 0.f;
+    uint32_t col;
+    bool live;
+    if (G >= 1 && cols <= TPB)
+    {
+        live = t < G * cols;
+        const uint32_t rsub = t / cols;
+        col = t - rsub * cols;
+        if (live)
+            for (size_t r = r_begin + rsub; r < r_end; r += G)
+            {
+                const size_t idx = r * cols + col;
+                float v = a[idx];
+                if (FUSED)
+                {
+                    v = g(act_ref[idx], v);
+                    dz[idx] = v;
+                }
+                acc += v;
+            }
+        lds[t] = acc;
+        __syncthreads();
+        if (t < cols)
+        {
+            float s = lds[t];
+            for (uint32_t q = 1; q < G; ++q)
+                s += lds[q * cols + t];
+            if (partial)
+                partial[(size_t)blockIdx.y * cols + t] = s;
+        }
+    }
+    else
+    {
+        col = blockIdx.x * TPB + t;
+        live = col < cols;
+        if (live)
+        {
+            for (size_t r = r_begin; r < r_end; ++r)
+            {
+                const size_t idx = r * cols + col;
+                float v = a[idx];
+                if (FUSED)
+                {
+                    v = g(act_ref[idx], v);
+                    dz[idx] = v;
+                }
+                acc += v;
+            }
+            if (partial)
+                partial[(size_t)blockIdx.y * cols + col] = acc;
+        }
+    }
+}
+
+__global__ __launch_bounds__(TPB) void colsum_stage2(const float* __restrict__ partial, float* __restrict__ out,
+                                                     uint32_t cols, uint32_t chunks)
+{
+    const uint32_t c = blockIdx.x * TPB + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.f;
+    for (uint32_t q = 0; q < chunks; ++q)
+        s += partial[(size_t)q * cols + c];
+    out[c] = s;
+}
+
+int run_colsum(const char* who, const float* a, const float* act_ref, float* dz, float* db, size_t rows,
+               size_t cols, ActGrad g, bool fused, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (cols == 0) return 0;
+    if (!a || (fused && (!act_ref || !dz))) return fail(DH_EINVAL, "%s: null tensor", who);
+    if (cols > 0x7fffffffu) return fail(DH_EINVAL, "%s: too many columns", who);
+    hipStream_t st = as_stream(stream);
+    if (rows == 0)
+    {
+        if (db)
+        {
+            hipLaunchKernelGGL(fill_zero, dim3(grid_for(cols)), dim3(TPB), 0, st, db, cols, false);
+            DH_LAUNCH_CHECK(who);
+        }
+        return 0;
+    }
+    const uint32_t G = cols <= TPB ? (uint32_t)(TPB / cols) : 0;
+    const unsigned col_tiles = cols <= TPB ? 1u : (unsigned)((cols + TPB - 1) / TPB);
+    // aim at ~4 workgroups per compute unit, at least 8 row groups each
+    size_t row_groups = G ? (rows + G - 1) / G : rows;
+    size_t chunks = ((size_t)num_cus() * 4 + col_tiles - 1) / col_tiles;
+    if (chunks > (row_groups + 7) / 8) chunks = (row_groups + 7) / 8;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 65535) chunks = 65535;
+    size_t rows_per_chunk = (rows + chunks - 1) / chunks;
+    if (G) rows_per_chunk = (rows_per_chunk + G - 1) / G * G;
+    chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
+    float* partial = nullptr;
+    if (db)
+    {
+        void* ws;
+        DH_TRY(workspace(chunks * cols * sizeof(float), &ws));
+        partial = static_cast<float*>(ws);
+    }
+    dim3 grid(col_tiles, (unsigned)chunks);
+    if (fused)
+        hipLaunchKernelGGL(colsum_stage1<true>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
+                           (uint32_t)cols, G, rows_per_chunk, g);
+    else
+        hipLaunchKernelGGL(colsum_stage1<false>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
+                           (uint32_t)cols, G, rows_per_chunk, g);
+    DH_LAUNCH_CHECK(who);
+    if (db)
+    {
+        hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + TPB - 1) / TPB)), dim3(TPB), 0, st, partial,
+                           db, (uint32_t)cols, (uint32_t)chunks);
+        DH_LAUNCH_CHECK(who);
+    }
+    return 0;
+}
+
+// ---- row sums: one wavefront per row -------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void rowsum_kernel(const float* __restrict__ a, float* __restrict__ out,
+                                                     size_t rows, size_t cols)
+{
+    const size_t row = (size_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows) return;
+    float s = 0.f;
+    for (size_t c = lane; c < cols; c += 64)
+        s += a[row * cols + c];
+    for (int off = 32; off > 0; off >>= 1)
+        s += __shfl_down(s, off, 64);
+    if (lane == 0) out[row] = s;
+}
+
+// ---- scalar reductions over short vectors (length = batch): one workgroup, fixed tree -------------
+struct RedSce
+{
+    __device__ float operator()(float y, float x) const
+    {
+        return x >= 0.f ? x - x * y + logf(1.f + expf(-x)) : -x * y + logf(1.f + expf(x));
+    }
+};
+struct RedMse
+{
+    __device__ float operator()(float y, float yh) const { return (y - yh) * (y - yh); }
+};
+
+template <class F>
+__global__ __launch_bounds__(1024) void mean_reduce(const float* __restrict__ a, const float* __restrict__ b,
+                                                    float* __restrict__ out, size_t n, F f)
+{
+    __shared__ float lds[1024];
+    float s = 0.f;
+    for (size_t i = threadIdx.x; i < n; i += 1024)
+        s += f(a[i], b[i]);
+    lds[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 512; w > 0; w >>= 1)
+    {
+        if ((int)threadIdx.x < w) lds[threadIdx.x] += lds[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = lds[0] / (float)n;
+}
+
+// rows whose first-maximum column agrees in y and y_hat (strict '>' keeps the lowest index on ties)
+__global__ __launch_bounds__(1024) void argmax_acc_kernel(const float* __restrict__ y, const float* __restrict__ yh,
+                                                          float* __restrict__ out, size_t rows, size_t cols)
+{
+    __shared__ unsigned int lds[1024];
+    unsigned int hits = 0;
+    for (size_t r = threadIdx.x; r < rows; r += 1024)
+    {
+        size_t by = 0, bh = 0;
+        for (size_t c = 1; c < cols; ++c)
+        {
+            if (y[r * cols + c] > y[r * cols + by]) by = c;
+            if (yh[r * cols + c] > yh[r * cols + bh]) bh = c;
+        }
+        hits += by == bh;
+    }
+    lds[threadIdx.x] = hits;
+    __syncthreads();
+    for (int w = 512; w > 0; w >>= 1)
+    {
+        if ((int)threadIdx.x < w) lds[threadIdx.x] += lds[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = (float)lds[0];
+}
+
+// ---- Adam ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void adam_update_kernel(float* __restrict__ p, const float* __restrict__ m,
+                                                          const float* __restrict__ v, float lrt, float eps, size_t n,
+                                                          bool vec)
+{
+    const size_t stride = (size_t)gridDim.x * TPB;
+    const size_t tid = (size_t)blockIdx.x * TPB + threadIdx.x;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride)
+        {
+            float4 pp = reinterpret_cast<float4*>(p)[i];
+            const float4 mm = reinterpret_cast<const float4*>(m)[i];
+            const float4 vv = reinterpret_cast<const float4*>(v)[i];
+            pp.x = pp.x - lrt * mm.x / (sqrtf(vv.x) + eps);
+            pp.y = pp.y - lrt * mm.y / (sqrtf(vv.y) + eps);
+            pp.z = pp.z - lrt * mm.z / (sqrtf(vv.z) + eps);
+            pp.w = pp.w - lrt * mm.w / (sqrtf(vv.w) + eps);
+            reinterpret_cast<float4*>(p)[i] = pp;
+        }
+        done = n4 * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride)
+        p[i] = p[i] - lrt * m[i] / (sqrtf(v[i]) + eps);
+}
+
+__device__ __forceinline__ void adam1(float& p, float& m, float& v, float g, float b1, float c1, float b2, float c2,
+                                      float lrt, float eps)
+{
+    m = b1 * m + c1 * g;
+    v = b2 * v + c2 * g * g;
+    p = p - lrt * m / (sqrtf(v) + eps);
+}
+
+__global__ __launch_bounds__(TPB) void adam_step_kernel(float* __restrict__ p, float* __restrict__ m, float* __restrict__ v,
+                                                        const float* __restrict__ g, float b1, float c1, float b2, float c2,
+                                                        float lrt, float eps, size_t n, bool vec)
+{
+    const size_t stride = (size_t)gridDim.x * TPB;
+    const size_t tid = (size_t)blockIdx.x * TPB + threadIdx.x;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t n4 = n / 4;
+        for (size_t i = tid; i < n4; i += stride)
+        {
+            float4 pp = reinterpret_cast<float4*>(p)[i];
+            float4 mm = reinterpret_cast<float4*>(m)[i];
+            float4 vv = reinterpret_cast<float4*>(v)[i];
+            const float4 gg = reinterpret_cast<const float4*>(g)[i];
+            adam1(pp.x, mm.x, vv.x, gg.x, b1, c1, b2, c2, lrt, eps);
+            adam1(pp.y, mm.y, vv.y, gg.y, b1, c1, b2, c2, lrt, eps);
+            adam1(pp.z, mm.z, vv.z, gg.z, b1, c1, b2, c2, lrt, eps);
+            adam1(pp.w, mm.w, vv.w, gg.w, b1, c1, b2, c2, lrt, eps);
+            reinterpret_cast<float4*>(p)[i] = pp;
+            reinterpret_cast<float4*>(m)[i] = mm;
+            reinterpret_cast<float4*>(v)[i] = vv;
+        }
+        done = n4 * 4;
+    }
+    for (size_t i = done + tid; i < n; i += stride)
+        adam1(p[i], m[i], v[i], g[i], b1, c1, b2, c2, lrt, eps);
+}
+
+__global__ __launch_bounds__(TPB) void sgd_update_kernel(float* __restrict__ var, const float* __restrict__ dv,
+                                                         const float* __restrict__ coeff, size_t n)
+{
+    const float c = coeff[0];
+    const size_t stride = (size_t)gridDim.x * TPB;
+    for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride)
+        var[i] += c * dv[i];
+}
+
+}  // namespace
+
+extern "C" {
+
+int dh_memset0(void* ptr, size_t bytes, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (bytes == 0) return 0;
+    if (!ptr || (bytes & 3) || (reinterpret_cast<uintptr_t>(ptr) & 3))
+        return fail(DH_EINVAL, "dh_memset0: pointer and size must be multiples of 4 bytes");
+    const size_t n = bytes / 4;
+    const bool vec = aligned16(ptr);
+    // a fill kernel rather than hipMemsetAsync, so that callers may capture it in a HIP graph
+    hipLaunchKernelGGL(fill_zero, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream),
+                       static_cast<float*>(ptr), n, vec);
+    DH_LAUNCH_CHECK("dh_memset0");
+    return 0;
+}
+
+int dh_bias_add(const float* z, const float* b, float* out, size_t rows, size_t cols, void* stream)
+{
+    DH_TRY(ensure_init());
+    const size_t n = rows * cols;
+    if (n == 0) return 0;
+    if (!z || !b || !out) return fail(DH_EINVAL, "dh_bias_add: null tensor");
+    if (n > 0x7fffffffu) return fail(DH_EINVAL, "dh_bias_add: more than 2^31-1 elements");
+    const bool vec = cols % 4 == 0 && aligned16(z) && aligned16(b) && aligned16(out);
+    const FastDiv fd((uint32_t)cols);
+    if (vec)
+        hipLaunchKernelGGL(bias_add_kernel<true>, dim3(grid_for(n / 4)), dim3(TPB), 0, as_stream(stream), z, b, out, n, fd);
+    else
+        hipLaunchKernelGGL(bias_add_kernel<false>, dim3(grid_for(n)), dim3(TPB), 0, as_stream(stream), z, b, out, n, fd);
+    DH_LAUNCH_CHECK("dh_bias_add");
+    return 0;
+}
+
+int dh_bias_grad(const float* dz, float* db, size_t rows, size_t cols, void* stream)
+{
+    if (!db && cols) return fail(DH_EINVAL, "dh_bias_grad: null result");
+    return run_colsum("dh_bias_grad", dz, nullptr, nullptr, db, rows, cols, ActGrad{DH_ACT_NONE, 0.f}, false, stream);
+}
+
+int dh_act_bias_grad(const float* act_ref, const float* dout, float* dz, float* db, size_t rows, size_t cols,
+                     int act, float alpha, void* stream)
+{
+    return run_colsum("dh_act_bias_grad", dout, act_ref, dz, db, rows, cols, ActGrad{act, alpha}, true, stream);
+}
+
+int dh_mat_sum_rows(const float* a, float* out, size_t rows, size_t cols, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (rows == 0) return 0;
+    if (!a || !out) return fail(DH_EINVAL, "dh_mat_sum_rows: null tensor");
+    hipLaunchKernelGGL(rowsum_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(TPB), 0, as_stream(stream), a, out, rows, cols);
+    DH_LAUNCH_CHECK("dh_mat_sum_rows");
+    return 0;
+}
+
+int dh_relu(const float* x, float* out, size_t n, void* stream) { return run_map1("dh_relu", x, out, n, stream, OpRelu{}); }
+int dh_relu_leaky(const float* x, float* out, size_t n, float alpha, void* stream)
+{ return run_map1("dh_relu_leaky", x, out, n, stream, OpLeaky{alpha}); }
+int dh_tanh(const float* x, float* out, size_t n, void* stream) { return run_map1("dh_tanh", x, out, n, stream, OpTanh{}); }
+int dh_sigmoid(const float* x, float* out, size_t n, void* stream) { return run_map1("dh_sigmoid", x, out, n, stream, OpSigmoid{}); }
+
+int dh_relu_grad(const float* z, const float* dout, float* out, size_t n, void* stream)
+{ return run_map2("dh_relu_grad", z, dout, out, n, stream, OpReluGrad{}); }
+int dh_leaky_relu_grad(const float* z, const float* dout, float* out, float alpha, size_t n, void* stream)
+{ return run_map2("dh_leaky_relu_grad", z, dout, out, n, stream, OpLeakyGrad{alpha}); }
+int dh_tanh_grad(const float* t, const float* dout, float* out, size_t n, void* stream)
+{ return run_map2("dh_tanh_grad", t, dout, out, n, stream, OpTanhGrad{}); }
+int dh_sigmoid_grad(const float* s, const float* dout, float* out, size_t n, void* stream)
+{ return run_map2("dh_sigmoid_grad", s, dout, out, n, stream, OpSigmoidGrad{}); }
+int dh_add(const float* a, const float* b, float* out, size_t n, void* stream)
+{ return run_map2("dh_add", a, b, out, n, stream, OpAdd{}); }
+
+int dh_sigmoid_cross_entropy(const float* y, const float* logits, float* out, size_t n, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (!y || !logits || !out || n == 0) return fail(DH_EINVAL, "dh_sigmoid_cross_entropy: null tensor or n == 0");
+    hipLaunchKernelGGL(mean_reduce<RedSce>, dim3(1), dim3(1024), 0, as_stream(stream), y, logits, out, n, RedSce{});
+    DH_LAUNCH_CHECK("dh_sigmoid_cross_entropy");
+    return 0;
+}
+
+int dh_sigmoid_cross_entropy_grad(const float* y, const float* logits, float* out, size_t n, void* stream)
+{ return run_map2("dh_sigmoid_cross_entropy_grad", y, logits, out, n, stream, OpSceGrad{1.f / (float)n}); }
+
+int dh_mse(const float* y, const float* y_hat, float* out, size_t rows, size_t cols, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (!y || !y_hat || !out || rows * cols == 0) return fail(DH_EINVAL, "dh_mse: null tensor or empty");
+    hipLaunchKernelGGL(mean_reduce<RedMse>, dim3(1), dim3(1024), 0, as_stream(stream), y, y_hat, out, rows * cols, RedMse{});
+    DH_LAUNCH_CHECK("dh_mse");
+    return 0;
+}
+
+int dh_mse_grad(const float* y, const float* y_hat, float* out, size_t n, void* stream)
+{ return run_map2("dh_mse_grad", y, y_hat, out, n, stream, OpMseGrad{(float)(2. / (double)n)}); }
+
+int dh_argmax_acc(const float* y, const float* y_hat, float* out, size_t rows, size_t cols, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (!y || !y_hat || !out || cols == 0) return fail(DH_EINVAL, "dh_argmax_acc: null tensor or no columns");
+    hipLaunchKernelGGL(argmax_acc_kernel, dim3(1), dim3(1024), 0, as_stream(stream), y, y_hat, out, rows, cols);
+    DH_LAUNCH_CHECK("dh_argmax_acc");
+    return 0;
+}
+
+int dh_moment_update(float* m, const float* g, float a, float b, size_t n, void* stream)
+{ return run_map2("dh_moment_update", m, g, m, n, stream, OpMoment{a, b}); }
+int dh_moment_update2(float* v, const float* g, float a, float b, size_t n, void* stream)
+{ return run_map2("dh_moment_update2", v, g, v, n, stream, OpMoment2{a, b}); }
+
+int dh_adam_update(float* p, const float* m, const float* v, float lrt, float eps, size_t n, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (n == 0) return 0;
+    if (!p || !m || !v) return fail(DH_EINVAL, "dh_adam_update: null tensor");
+    const bool vec = aligned16(p) && aligned16(m) && aligned16(v);
+    hipLaunchKernelGGL(adam_update_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), p, m, v,
+                       lrt, eps, n, vec);
+    DH_LAUNCH_CHECK("dh_adam_update");
+    return 0;
+}
+
+int dh_adam_step(float* p, float* m, float* v, const float* g, float beta1, float beta2, float lrt, float eps,
+                 size_t n, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (n == 0) return 0;
+    if (!p || !m || !v || !g) return fail(DH_EINVAL, "dh_adam_step: null tensor");
+    const bool vec = aligned16(p) && aligned16(m) && aligned16(v) && aligned16(g);
+    // 1 - beta in float, as src/api/adam-optimizer.cu forms the second coefficient
+    hipLaunchKernelGGL(adam_step_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), p, m, v, g,
+                       beta1, 1.f - beta1, beta2, 1.f - beta2, lrt, eps, n, vec);
+    DH_LAUNCH_CHECK("dh_adam_step");
+    return 0;
+}
+
+int dh_sgd_update(float* var, const float* dv, const float* coeff_device, size_t n, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (n == 0) return 0;
+    if (!var || !dv || !coeff_device) return fail(DH_EINVAL, "dh_sgd_update: null tensor");
+    hipLaunchKernelGGL(sgd_update_kernel, dim3(grid_for(n)), dim3(TPB), 0, as_stream(stream), var, dv, coeff_device, n);
+    DH_LAUNCH_CHECK("dh_sgd_update");
+    return 0;
+}
+
+}

@@ -1,0 +1,237 @@
+// Runtime half of the C ABI: device selection, memory, streams, events and the scratch arena.
+// Stands in for the GPU branches of the reference's src/memory (alloc.cu, copy.hxx).
+#include "dh_common.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+namespace dh
+{
+namespace
+{
+thread_local char g_err[512] = "";
+
+struct DeviceState
+{
+    bool ready = false;
+    int device = 0;
+    int cus = 0;
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+};
+
+std::mutex g_mu;
+DeviceState g_dev[16];
+int g_cur = -1;
+}  // namespace
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int fail_hip(hipError_t err, const char* what)
+{
+    return fail((int)err, "%s: %s (%s)", what, hipGetErrorString(err), hipGetErrorName(err));
+}
+
+static int init_device(int device)
+{
+    if (device < 0 || device >= 16)
+        return fail(DH_EINVAL, "dh_init: device %d out of range", device);
+    std::lock_guard<std::mutex> lock(g_mu);
+    DH_HIP(hipSetDevice(device));
+    DeviceState& st = g_dev[device];
+    if (!st.ready)
+    {
+        hipDeviceProp_t prop;
+        DH_HIP(hipGetDeviceProperties(&prop, device));
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            return fail(DH_EINVAL, "dh_init: device %d is %s; this library holds gfx950 code only",
+                        device, prop.gcnArchName);
+        st.device = device;
+        st.cus = prop.multiProcessorCount;
+        st.ready = true;
+    }
+    g_cur = device;
+    return 0;
+}
+
+int ensure_init()
+{
+    if (g_cur >= 0)
+        return 0;
+    return init_device(0);
+}
+
+int num_cus()
+{
+    return g_cur >= 0 ? g_dev[g_cur].cus : 256;
+}
+
+int workspace(size_t bytes, void** ptr)
+{
+    DH_TRY(ensure_init());
+    std::lock_guard<std::mutex> lock(g_mu);
+    DeviceState& st = g_dev[g_cur];
+    if (bytes > st.ws_bytes)
+    {
+        // Work queued on the old arena must drain before it is released.
+        DH_HIP(hipDeviceSynchronize());
+        if (st.ws)
+            DH_HIP(hipFree(st.ws));
+        st.ws = nullptr;
+        st.ws_bytes = 0;
+        size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+        DH_HIP(hipMalloc(&st.ws, want));
+        st.ws_bytes = want;
+    }
+    *ptr = st.ws;
+    return 0;
+}
+
+}  // namespace dh
+
+using namespace dh;
+
+extern "C" {
+
+const char* dh_version(void) { return "dcgan_hip 0.1 (gfx950)"; }
+
+const char* dh_last_error(void) { return g_err; }
+
+int dh_init(int device) { return init_device(device); }
+
+int dh_device_info(char* name, size_t name_len, int* compute_units, int* clock_khz,
+                   size_t* memory_bytes)
+{
+    DH_TRY(ensure_init());
+    hipDeviceProp_t prop;
+    DH_HIP(hipGetDeviceProperties(&prop, g_cur));
+    if (name && name_len)
+    {
+        snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    if (memory_bytes) *memory_bytes = prop.totalGlobalMem;
+    return 0;
+}
+
+int dh_malloc(void** ptr, size_t bytes)
+{
+    DH_TRY(ensure_init());
+    if (!ptr) return fail(DH_EINVAL, "dh_malloc: null result pointer");
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 4;
+    DH_HIP(hipMalloc(ptr, bytes));
+    return 0;
+}
+
+int dh_free(void* ptr)
+{
+    if (!ptr) return 0;
+    DH_TRY(ensure_init());
+    DH_HIP(hipFree(ptr));
+    return 0;
+}
+
+int dh_memcpy_h2d(void* dst, const void* src, size_t bytes)
+{
+    DH_TRY(ensure_init());
+    if (bytes == 0) return 0;
+    DH_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int dh_memcpy_d2h(void* dst, const void* src, size_t bytes)
+{
+    DH_TRY(ensure_init());
+    if (bytes == 0) return 0;
+    DH_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int dh_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (bytes == 0) return 0;
+    DH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return 0;
+}
+
+int dh_sync(void)
+{
+    DH_TRY(ensure_init());
+    DH_HIP(hipDeviceSynchronize());
+    return 0;
+}
+
+int dh_stream_create(void** stream)
+{
+    DH_TRY(ensure_init());
+    hipStream_t s;
+    DH_HIP(hipStreamCreate(&s));
+    *stream = s;
+    return 0;
+}
+
+int dh_stream_destroy(void* stream)
+{
+    DH_HIP(hipStreamDestroy(as_stream(stream)));
+    return 0;
+}
+
+int dh_stream_sync(void* stream)
+{
+    DH_TRY(ensure_init());
+    DH_HIP(hipStreamSynchronize(as_stream(stream)));
+    return 0;
+}
+
+int dh_event_create(void** event)
+{
+    DH_TRY(ensure_init());
+    hipEvent_t e;
+    DH_HIP(hipEventCreate(&e));
+    *event = e;
+    return 0;
+}
+
+int dh_event_destroy(void* event)
+{
+    DH_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return 0;
+}
+
+int dh_event_record(void* event, void* stream)
+{
+    DH_HIP(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+    return 0;
+}
+
+int dh_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+    DH_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+    DH_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return 0;
+}
+
+int dh_workspace_reserve(size_t bytes)
+{
+    void* p;
+    return workspace(bytes, &p);
+}
+
+size_t dh_workspace_bytes(void)
+{
+    return g_cur >= 0 ? g_dev[g_cur].ws_bytes : 0;
+}
+
+}

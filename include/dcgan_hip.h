@@ -1,0 +1,186 @@
+/*
+ * dcgan_hip.h -- C ABI of the MI355X (gfx950) backend for dcgan-cuda's convolution hot path.
+ *
+ * One entry point per operator of the reference's GPU kernel table (src/gpu/kernels.cu:23-61)
+ * that a DCGAN training iteration reaches, plus the memory calls behind the reference's
+ * tensor_alloc / tensor_write / tensor_read (src/memory/alloc.cu, src/memory/copy.hxx).
+ * Plain pointers and sizes only: every `float*` is a DEVICE pointer unless the comment says
+ * host.  All tensors are fp32; activations NHWC, filters HWIO, matrices row-major -- the
+ * reference's layouts.  `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ * calls are asynchronous with respect to the host unless stated otherwise.
+ *
+ * Every function returns 0 on success or a non-zero code (a hipError_t value, or DH_EINVAL for
+ * arguments the kernels cannot take); dh_last_error() describes the last failure of the calling
+ * thread.  The host shim turns non-zero into std::runtime_error, the reference's convention
+ * (src/memory/alloc.cu:6-14).
+ *
+ * Each declaration cites the reference interface it stands in for.
+ */
+#ifndef DCGAN_HIP_H
+#define DCGAN_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DH_EINVAL 10001
+
+/* Epilogue activations that the convolution entry points can fuse. */
+enum { DH_ACT_NONE = 0, DH_ACT_RELU = 1, DH_ACT_LEAKY = 2, DH_ACT_TANH = 3, DH_ACT_SIGMOID = 4 };
+
+/* ---- runtime / memory ---------------------------------------------------------------------- */
+
+/* Library version string. */
+const char* dh_version(void);
+/* Message of the last failed call on this thread ("" if none). */
+const char* dh_last_error(void);
+/* Select the GPU and create the library's state on it.  Optional: the first call of any other
+ * function initialises device 0.  (The reference has no explicit init: its first cudaMalloc,
+ * src/memory/alloc.cu:20, creates the context.) */
+int dh_init(int device);
+/* Name, compute-unit count, engine clock (kHz) and memory size of the current device. */
+int dh_device_info(char* name, size_t name_len, int* compute_units, int* clock_khz,
+                   size_t* memory_bytes);
+/* tensor_alloc / tensor_free in GPU mode: src/memory/alloc.cu:16-37 (cudaMalloc / cudaFree). */
+int dh_malloc(void** ptr, size_t bytes);
+int dh_free(void* ptr);
+/* tensor_write / tensor_read in GPU mode: src/memory/copy.hxx:29-46 (blocking cudaMemcpy). */
+int dh_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
+int dh_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
+int dh_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
+/* tensor_fill with zero (src/memory/copy.hxx:7-27) without the host staging buffer. */
+int dh_memset0(void* ptr, size_t bytes, void* stream);
+/* cudaDeviceSynchronize of src/gpu/runner.cu:16, moved out of the per-node loop. */
+int dh_sync(void);
+int dh_stream_create(void** stream);
+int dh_stream_destroy(void* stream);
+int dh_stream_sync(void* stream);
+/* HIP events for timing on the stream the kernels run on. */
+int dh_event_create(void** event);
+int dh_event_destroy(void* event);
+int dh_event_record(void* event, void* stream);
+int dh_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+/* Split-K partial sums live in a per-device scratch arena that grows on demand; reserving the
+ * largest size up front keeps hipMalloc out of the steady state.  (Replaces the 3-4
+ * cudaMalloc/cudaFree per call of src/gpu/conv2d_gemm.hh:514-553.) */
+int dh_workspace_reserve(size_t bytes);
+size_t dh_workspace_bytes(void);
+
+/* ---- convolutions: fp32 implicit GEMM on MFMA, no im2col buffer ------------------------------ */
+
+/* conv2d forward, optionally with the bias add and activation that follow it fused in.
+ * Replaces gpu::kernel_conv2d (src/gpu/conv2d.cu:13-62) [+ mvrow_add, src/gpu/matmul.cu:28-38,
+ * + vect_relu_leaky etc., src/gpu/relu.cu:26-55].  Also serves conv2d_transpose's input
+ * gradient (src/gpu/conv2d.cu:214-259).
+ *   x [N,H,W,C]  k [kh,kw,C,O]  y [N,Ho,Wo,O]
+ *   y[b,i,j,o] = act(bias[o] + sum_{di,dj,c} x[b, sh*i+di-pad_top, sw*j+dj-pad_left, c] * k[di,dj,c,o])
+ * pad_top / pad_left are the pads BEFORE the image (the reference's pad_total / 2).
+ * bias may be NULL; alpha is the leaky slope. */
+int dh_conv2d_fwd(const float* x, const float* k, float* y,
+                  int N, int H, int W, int C, int kh, int kw, int O,
+                  int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,
+                  const float* bias, int act, float alpha, void* stream);
+
+/* conv2d input gradient == conv2d_transpose forward, optionally with bias + activation fused.
+ * Replaces gpu::kernel_conv2d_input_grad (src/gpu/conv2d.cu:70-117) and
+ * gpu::kernel_conv2d_transpose (src/gpu/conv2d.cu:167-212).
+ *   dy [N,Ho,Wo,O]  k [kh,kw,C,O]  dx [N,H,W,C]
+ *   dx[b,h,w,c] = act(bias[c] + sum over (i,di): sh*i+di-pad_top == h, (j,dj) likewise, o of
+ *                 dy[b,i,j,o] * k[di,dj,c,o])
+ * pad_top / pad_left are those of the forward convolution this is the adjoint of. */
+int dh_conv2d_dx(const float* dy, const float* k, float* dx,
+                 int N, int Ho, int Wo, int O, int kh, int kw, int C,
+                 int sh, int sw, int pad_top, int pad_left, int H, int W,
+                 const float* bias, int act, float alpha, void* stream);
+
+/* conv2d filter gradient.  Replaces gpu::kernel_conv2d_kernel_grad (src/gpu/conv2d.cu:119-165)
+ * and, with the roles of the activations exchanged, gpu::kernel_conv2d_transpose_kernel_grad
+ * (src/gpu/conv2d.cu:264-307).
+ *   x [N,H,W,C]  dy [N,Ho,Wo,O]  dk [kh,kw,C,O]
+ *   dk[di,dj,c,o] = sum_{b,i,j} x[b, sh*i+di-pad_top, sw*j+dj-pad_left, c] * dy[b,i,j,o]
+ * Split-K partial sums are reduced in a fixed order: results are reproducible run to run. */
+int dh_conv2d_dk(const float* x, const float* dy, float* dk,
+                 int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw,
+                 int sh, int sw, int pad_top, int pad_left, void* stream);
+
+/* ---- bias and activations: coalesced, vectorised, one pass over HBM ----------------------------- */
+
+/* out[r,c] = z[r,c] + b[c].  conv2d_bias_add lowers to this (src/ops/conv2d-bias-add.cu:35-38);
+ * replaces gpu::mvrow_add (src/gpu/matmul.cu:28-38, :106-119). */
+int dh_bias_add(const float* z, const float* b, float* out, size_t rows, size_t cols, void* stream);
+/* db[c] = sum_r dz[r,c].  conv2d_bias_add_grad lowers to this
+ * (src/ops/conv2d-bias-add-grad.cu:29-31); replaces gpu::mat_sum_cols (src/gpu/sum.cu:112-151). */
+int dh_bias_grad(const float* dz, float* db, size_t rows, size_t cols, void* stream);
+/* out[r] = sum_c a[r,c].  Replaces gpu::mat_sum_rows (src/gpu/sum.cu:69-108). */
+int dh_mat_sum_rows(const float* a, float* out, size_t rows, size_t cols, void* stream);
+/* Replace vect_relu / vect_relu_leaky (src/gpu/relu.cu:26-55), vect_sigmoid / vect_tanh
+ * (src/gpu/sigmoid.cu:22-50). */
+int dh_relu(const float* x, float* out, size_t n, void* stream);
+int dh_relu_leaky(const float* x, float* out, size_t n, float alpha, void* stream);
+int dh_tanh(const float* x, float* out, size_t n, void* stream);
+int dh_sigmoid(const float* x, float* out, size_t n, void* stream);
+/* Replace vect_relu_grad / vect_relu_leaky_grad (src/gpu/relu.cu:36-66), vect_sigmoid_grad and
+ * vect_tanh_grad (src/gpu/sigmoid.cu:32-40, :114-122).  relu_grad passes dout where z > 0,
+ * leaky_relu_grad scales dout by alpha where z < 0; tanh/sigmoid gradients take the forward
+ * OUTPUT. */
+int dh_relu_grad(const float* z, const float* dout, float* out, size_t n, void* stream);
+int dh_leaky_relu_grad(const float* z, const float* dout, float* out, float alpha, size_t n, void* stream);
+int dh_tanh_grad(const float* tanh_out, const float* dout, float* out, size_t n, void* stream);
+int dh_sigmoid_grad(const float* sig_out, const float* dout, float* out, size_t n, void* stream);
+/* out = a + b.  Replaces gpu::vect_add (src/gpu/sum.cu:207-214). */
+int dh_add(const float* a, const float* b, float* out, size_t n, void* stream);
+/* Fused backward step of a conv layer's bias/activation pair: dz = act'(.) * dout and
+ * db[c] = sum_r dz[r,c] in one pass.  `act_ref` is z for relu/leaky (the forward output works
+ * equally: same sign) and the forward output for tanh/sigmoid.  db may be NULL.
+ * Fuses leaky_relu_grad + mat_sum_cols of the reference's backward node list. */
+int dh_act_bias_grad(const float* act_ref, const float* dout, float* dz, float* db,
+                     size_t rows, size_t cols, int act, float alpha, void* stream);
+
+/* ---- losses --------------------------------------------------------------------------------------- */
+
+/* *out = mean_i( x>=0 ? x - x*y + log(1+exp(-x)) : -x*y + log(1+exp(x)) ); out is a device scalar.
+ * Replaces gpu::sigmoid_cross_entropy (src/gpu/sigmoid.cu:61-100). */
+int dh_sigmoid_cross_entropy(const float* y, const float* logits, float* out, size_t n, void* stream);
+/* out[i] = (sigmoid(x[i]) - y[i]) / n.  Replaces src/gpu/sigmoid.cu:103-111. */
+int dh_sigmoid_cross_entropy_grad(const float* y, const float* logits, float* out, size_t n, void* stream);
+/* Mean squared error and its gradient 2/n*(y_hat - y), the loss the reference's conv-gradient tests
+ * use (tests/test_conv2d_grad.cu:96).  Replace gpu::mse / mse_grad (src/gpu/sum.cu:15-65). */
+int dh_mse(const float* y, const float* y_hat, float* out, size_t rows, size_t cols, void* stream);
+int dh_mse_grad(const float* y, const float* y_hat, float* out, size_t n, void* stream);
+/* *out = number of rows whose first-maximum column agrees in y and y_hat (ties -> lowest index).
+ * Replaces gpu::argmax_acc (src/gpu/sum.cu:154-204). */
+int dh_argmax_acc(const float* y, const float* y_hat, float* out, size_t rows, size_t cols, void* stream);
+
+/* ---- dense layers --------------------------------------------------------------------------------- */
+
+/* out (m x p) = a (m x n) * b (n x p) [+ bias (p)].  Replace gpu::matmul / matmul_add
+ * (src/gpu/matmul.cu:12-26, :40-56). */
+int dh_gemm_nn(const float* a, const float* b, const float* bias, float* out,
+               size_t m, size_t n, size_t p, void* stream);
+/* out (m x p) = tr(a) * b, a is (n x m), b is (n x p).  Replaces tmat_mat_mul (src/gpu/matmul.cu:58-71). */
+int dh_gemm_tn(const float* a, const float* b, float* out, size_t m, size_t n, size_t p, void* stream);
+/* out (m x p) = a * tr(b), a is (m x n), b is (p x n).  Replaces mat_tmat_mul (src/gpu/matmul.cu:73-86). */
+int dh_gemm_nt(const float* a, const float* b, float* out, size_t m, size_t n, size_t p, void* stream);
+
+/* ---- optimisers: single pass, HBM-bandwidth bound --------------------------------------------------- */
+
+/* m = a*m + b*g.  Replaces gpu::moment_update (src/gpu/update.cu:24-32). */
+int dh_moment_update(float* m, const float* g, float a, float b, size_t n, void* stream);
+/* v = a*v + b*g*g.  Replaces gpu::moment_update2 (src/gpu/update.cu:35-43). */
+int dh_moment_update2(float* v, const float* g, float a, float b, size_t n, void* stream);
+/* p -= lrt * m / (sqrt(v) + eps); lrt = lr*sqrt(1-beta2^t)/(1-beta1^t) is formed by the caller on
+ * the host in float, as the reference does (src/gpu/update.cu:81-96). */
+int dh_adam_update(float* p, const float* m, const float* v, float lrt, float eps, size_t n, void* stream);
+/* The three kernels above in one pass (28 B/param instead of 40): m, v and p are updated in place
+ * with the same arithmetic, in the same order, as the three separate calls. */
+int dh_adam_step(float* p, float* m, float* v, const float* g, float beta1, float beta2,
+                 float lrt, float eps, size_t n, void* stream);
+/* var += *coeff * dv with coeff a DEVICE scalar.  Replaces gpu::vect_update (src/gpu/update.cu:14-21). */
+int dh_sgd_update(float* var, const float* dv, const float* coeff_device, size_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,119 @@
+"""Convolution kernels against the CPU oracle on seeded inputs: odd shapes that exercise every
+bounds check and the scalar-load paths, DCGAN layer shapes at a small batch, fused epilogues, and
+split-K.  Tolerance: 1e-4 relative / 1e-5 absolute (fp32), scaled by the magnitude of the
+reduction for the filter gradient whose sums run over the whole batch."""
+import numpy as np
+import pytest
+
+from common import RTOL, ATOL, rand_conv_inputs, same_pad
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [  # N, H, W, C, kh, kw, O, stride
+    (2, 8, 8, 3, 5, 5, 4, 2),
+    (1, 7, 9, 2, 3, 3, 5, 2),
+    (2, 6, 6, 4, 5, 5, 3, 1),
+    (1, 9, 7, 2, 3, 5, 2, 3),
+    (3, 4, 4, 8, 2, 2, 8, 2),
+    (1, 5, 5, 1, 5, 5, 1, 2),
+    (2, 11, 13, 12, 3, 3, 20, 1),
+    (1, 10, 10, 16, 1, 1, 8, 3),      # 1x1 filter, stride 3: dx phases without any tap
+    (5, 12, 12, 36, 5, 5, 72, 2),     # vector loads with partial tiles
+    (2, 32, 32, 64, 5, 5, 128, 2),    # D1 at batch 2
+    (2, 16, 16, 128, 5, 5, 256, 2),   # D2 at batch 2
+    (4, 8, 8, 256, 5, 5, 512, 2),     # D3 at batch 4 (split-K)
+    (2, 64, 64, 3, 5, 5, 64, 2),      # D0 at batch 2
+]
+
+
+@pytest.fixture(scope="module")
+def be():
+    import __graft_entry__ as ge
+    return ge.load_package().HipBackend(0)
+
+
+def close(got, exp, scale=1.0, what=""):
+    np.testing.assert_allclose(got, exp, rtol=RTOL, atol=ATOL * scale, err_msg=what)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_conv_fwd_dx_dk(be, orc, shape):
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(42, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    orc.set_threads(8)
+    close(be.conv2d(x, k, (s, s)), orc.conv2d(x, k, (s, s)), what="fwd")
+    close(be.conv2d_input_grad(dy, k, s, (H, W)), orc.conv2d_input_grad(dy, k, s, (H, W)), what="dx")
+    exp = orc.conv2d_kernel_grad(dy, x, s, pads)
+    # sums of N*Ho*Wo products of U(-1,1) values: absolute tolerance follows their magnitude
+    close(be.conv2d_kernel_grad(dy, x, s, pads), exp, scale=max(1.0, float(np.abs(exp).max())), what="dk")
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 4, 512, 5, 5, 256, 2), (2, 32, 32, 64, 5, 5, 3, 2), (3, 5, 7, 6, 3, 3, 4, 2)])
+def test_conv_transpose_and_grads(be, orc, shape):
+    """Generator-style layers: x [N,Hi,Wi,Ci] -> [N,s*Hi,s*Wi,Co], filter [kh,kw,Co,Ci]."""
+    print("shape", shape, flush=True)
+    N, Hi, Wi, Ci, kh, kw, Co, s = shape
+    rng = np.random.default_rng(17)
+    x = rng.uniform(-1, 1, (N, Hi, Wi, Ci)).astype(np.float32)
+    k = (rng.standard_normal((kh, kw, Co, Ci)) * 0.02).astype(np.float32)
+    dy = rng.uniform(-1, 1, (N, Hi * s, Wi * s, Co)).astype(np.float32)
+    orc.set_threads(8)
+    close(be.conv2d_transpose(x, k, (Hi * s, Wi * s), s), orc.conv2d_transpose(x, k, (Hi * s, Wi * s), s))
+    close(be.conv2d_transpose_input_grad(dy, k, s, (Hi, Wi)), orc.conv2d_transpose_input_grad(dy, k, s, (Hi, Wi)))
+    exp = orc.conv2d_transpose_kernel_grad(dy, x, s, (kh, kw))
+    close(be.conv2d_transpose_kernel_grad(dy, x, s, (kh, kw)), exp, scale=max(1.0, float(np.abs(exp).max())))
+
+
+@pytest.mark.parametrize("act", ["none", "relu", "leaky", "tanh", "sigmoid"])
+@pytest.mark.parametrize("shape", [(2, 16, 16, 32, 5, 5, 64, 2), (4, 8, 8, 256, 5, 5, 512, 2), (1, 7, 9, 2, 3, 3, 5, 2)])
+def test_fused_epilogues(be, orc, act, shape):
+    """conv + bias + activation in one call == the three reference operators in sequence;
+    the second shape takes the split-K path, where the epilogue runs in the reduction."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(5, *shape)
+    rng = np.random.default_rng(1)
+    code = {"none": A.ACT_NONE, "relu": A.ACT_RELU, "leaky": A.ACT_LEAKY, "tanh": A.ACT_TANH, "sigmoid": A.ACT_SIGMOID}[act]
+    f = {"none": lambda v: v, "relu": orc.relu, "leaky": lambda v: orc.relu_leaky(v, 0.2), "tanh": orc.tanh,
+         "sigmoid": orc.sigmoid}[act]
+    b = (rng.standard_normal(O) * 0.5).astype(np.float32)
+    close(be.conv2d(x, k, (s, s), bias=b, act=code, alpha=0.2), f(orc.bias_add(orc.conv2d(x, k, (s, s)), b)))
+    bc = (rng.standard_normal(C) * 0.5).astype(np.float32)
+    close(be.conv2d_input_grad(dy, k, s, (H, W), bias=bc, act=code, alpha=0.2),
+          f(orc.bias_add(orc.conv2d_input_grad(dy, k, s, (H, W)), bc)))
+
+
+def test_dk_is_reproducible(be):
+    """Split-K partial sums are reduced in a fixed order: two runs give identical bits."""
+    x, k, dy = rand_conv_inputs(3, 8, 16, 16, 128, 5, 5, 256, 2)
+    a = be.conv2d_kernel_grad(dy, x, 2, (3, 3))
+    b = be.conv2d_kernel_grad(dy, x, 2, (3, 3))
+    np.testing.assert_array_equal(a, b)
+
+
+def test_adjoint_at_full_batch(be):
+    """Size-independent check at the benchmark's batch 64 (where the CPU oracle would take minutes):
+    <conv(x,k), dy> = <x, dx(dy,k)> = <k, dk(x,dy)> for layer D2."""
+    shape = (64, 16, 16, 128, 5, 5, 256, 2)
+    x, k, dy = rand_conv_inputs(9, *shape)
+    y = be.conv2d(x, k, (2, 2)).astype(np.float64)
+    lhs = np.vdot(y, dy)
+    a = np.vdot(x.astype(np.float64), be.conv2d_input_grad(dy, k, 2, (16, 16)))
+    b = np.vdot(k.astype(np.float64), be.conv2d_kernel_grad(dy, x, 2, (3, 3)))
+    assert abs(lhs - a) <= 1e-4 * abs(lhs) + 1e-2
+    assert abs(lhs - b) <= 1e-4 * abs(lhs) + 1e-2
+
+
+def test_bad_arguments_are_rejected(be):
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    x = A.Buf((1, 4, 4, 1))
+    with pytest.raises(A.HipError):
+        A.check(be.lib.dh_conv2d_fwd(x.ptr, x.ptr, x.ptr, 1, 4, 4, 1, 2, 2, 1, 2, 2, 5, 0, 2, 2, None, 0, 0.0, None))
+    with pytest.raises(A.HipError):
+        A.check(be.lib.dh_conv2d_fwd(None, x.ptr, x.ptr, 1, 4, 4, 1, 2, 2, 1, 2, 2, 0, 0, 2, 2, None, 0, 0.0, None))
+    with pytest.raises(A.HipError):
+        A.check(be.lib.dh_conv2d_dk(x.ptr, x.ptr, x.ptr, 0, 4, 4, 1, 2, 2, 1, 2, 2, 2, 2, 0, 0, None))

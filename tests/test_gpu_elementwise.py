@@ -1,0 +1,125 @@
+"""Bias, activation, loss, dense and Adam kernels against the CPU oracle at sizes that cover the
+vector path, the scalar tail, the narrow (3-channel) and wide (512 / 8192 column) reductions."""
+import numpy as np
+import pytest
+
+from common import RTOL, ATOL
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def be():
+    import __graft_entry__ as ge
+    return ge.load_package().HipBackend(0)
+
+
+def close(got, exp, scale=1.0):
+    np.testing.assert_allclose(got, exp, rtol=RTOL, atol=ATOL * scale)
+
+
+@pytest.mark.parametrize("n", [1, 3, 255, 1024, 4099, 786432])
+def test_activations_and_grads(be, orc, n):
+    rng = np.random.default_rng(n)
+    a = rng.uniform(-4, 4, n).astype(np.float32)
+    d = rng.uniform(-1, 1, n).astype(np.float32)
+    a[:1] = 0.0
+    np.testing.assert_array_equal(be.relu(a), orc.relu(a))
+    np.testing.assert_array_equal(be.relu_leaky(a, 0.2), orc.relu_leaky(a, 0.2))
+    np.testing.assert_array_equal(be.relu_grad(a, d), orc.relu_grad(a, d))
+    np.testing.assert_array_equal(be.leaky_relu_grad(a, d, 0.2), orc.leaky_relu_grad(a, d, 0.2))
+    close(be.tanh(a), orc.tanh(a))
+    close(be.sigmoid(a), orc.sigmoid(a))
+    t, s = orc.tanh(a), orc.sigmoid(a)
+    close(be.tanh_grad(t, d), orc.tanh_grad(t, d))
+    close(be.sigmoid_grad(s, d), orc.sigmoid_grad(s, d))
+    np.testing.assert_array_equal(be.add(a, d), orc.add(a, d))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 3), (4096, 3), (1000, 64), (333, 128), (64, 512), (64, 8192), (5, 300), (4097, 20)])
+def test_bias_add_and_grad(be, orc, rows, cols):
+    rng = np.random.default_rng(rows * 31 + cols)
+    z = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    b = rng.standard_normal(cols).astype(np.float32)
+    np.testing.assert_array_equal(be.bias_add(z, b), orc.bias_add(z, b))
+    exp = orc.bias_grad(z)
+    close(be.bias_grad(z), exp, scale=max(1.0, np.sqrt(rows)))
+    close(be.mat_sum_rows(z), orc.mat_sum_rows(z), scale=max(1.0, np.sqrt(cols)))
+
+
+@pytest.mark.parametrize("act", ["relu", "leaky", "tanh", "none"])
+@pytest.mark.parametrize("rows,cols", [(2048, 64), (1031, 3), (64, 512)])
+def test_fused_act_bias_grad(be, orc, act, rows, cols):
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    rng = np.random.default_rng(7)
+    z = rng.uniform(-2, 2, (rows, cols)).astype(np.float32)
+    d = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    if act == "relu":
+        ref, dz, code = orc.relu(z), orc.relu_grad(z, d), A.ACT_RELU          # forward OUTPUT as reference
+    elif act == "leaky":
+        ref, dz, code = orc.relu_leaky(z, 0.2), orc.leaky_relu_grad(z, d, 0.2), A.ACT_LEAKY
+    elif act == "tanh":
+        ref = orc.tanh(z)
+        dz, code = orc.tanh_grad(ref, d), A.ACT_TANH
+    else:
+        ref, dz, code = z, d, A.ACT_NONE
+    got_dz, got_db = be.act_bias_grad(ref, d, code, 0.2)
+    close(got_dz, dz)
+    close(got_db, orc.bias_grad(dz), scale=max(1.0, np.sqrt(rows)))
+
+
+def test_losses(be, orc):
+    rng = np.random.default_rng(2)
+    for n in (1, 64, 512, 5000):
+        x = rng.uniform(-6, 6, n).astype(np.float32)
+        y = (rng.uniform(0, 1, n) > 0.5).astype(np.float32)
+        close(be.sigmoid_cross_entropy(y, x), orc.sigmoid_cross_entropy(y, x))
+        close(be.sigmoid_cross_entropy_grad(y, x), orc.sigmoid_cross_entropy_grad(y, x))
+    a = rng.uniform(-1, 1, (16, 40)).astype(np.float32)
+    b = rng.uniform(-1, 1, (16, 40)).astype(np.float32)
+    close(be.mse(a, b), orc.mse(a, b))
+    close(be.mse_grad(a, b), orc.mse_grad(a, b))
+
+
+def test_argmax_is_exact(be, orc):
+    rng = np.random.default_rng(4)
+    for rows, cols in ((10, 3), (64, 10), (1500, 7), (3, 1)):
+        y = rng.uniform(0, 1, (rows, cols)).astype(np.float32)
+        yh = rng.uniform(0, 1, (rows, cols)).astype(np.float32)
+        yh[::2] = y[::2]
+        y[1, :] = 0.5   # ties -> lowest index on both sides
+        assert be.argmax_acc(y, yh) == orc.argmax_acc(y, yh)
+
+
+@pytest.mark.parametrize("m,n,p", [(64, 100, 8192), (64, 8192, 1), (9, 33, 17), (1, 1, 1), (130, 70, 65)])
+def test_dense(be, orc, m, n, p):
+    rng = np.random.default_rng(m + n + p)
+    x = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    w = (rng.standard_normal((n, p)) * 0.02).astype(np.float32)
+    b = rng.standard_normal(p).astype(np.float32)
+    g = rng.uniform(-1, 1, (m, p)).astype(np.float32)
+    orc.set_threads(8)
+    close(be.mat_mul_add(x, w, b), orc.mat_mul_add(x, w, b))
+    close(be.mm_mul(x, w), orc.mm_mul(x, w))
+    close(be.tmm_mul(x, g), orc.tmm_mul(x, g), scale=4)    # tr(x) g : dW
+    close(be.mtm_mul(g, w), orc.mtm_mul(g, w))             # g tr(w) : dx
+
+
+@pytest.mark.parametrize("n", [1, 1000, 4099, 3276800])
+def test_adam(be, orc, n):
+    rng = np.random.default_rng(n)
+    p = rng.standard_normal(n).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    m = rng.standard_normal(n).astype(np.float32) * 0.1
+    v = rng.uniform(0, 1, n).astype(np.float32) * 0.01
+    em, ev = orc.moment_update(m, g, 0.5, 0.5), orc.moment_update2(v, g, 0.999, 0.001)
+    close(be.moment_update(m, g, 0.5, 0.5), em)
+    close(be.moment_update2(v, g, 0.999, 0.001), ev)
+    t, lrt = orc.adam_lrt(0, 2e-4, 0.5, 0.999)
+    ep = orc.adam_apply(p, em, ev, lrt, 1e-8)
+    close(be.adam_apply(p, em, ev, lrt, 1e-8), ep)
+    # the fused single-pass step equals the three separate operators
+    gp, gm, gv = be.adam_step(p, m, v, g, 0.5, 0.999, lrt, 1e-8)
+    close(gm, em), close(gv, ev), close(gp, ep)
+    close(be.vect_update(p, g, -0.1), orc.vect_update(p, g, -0.1))
