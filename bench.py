@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the convolution hot path on one MI355X.
+
+One "step" is one full DCGAN training iteration at batch 64 in fp32 (BASELINE.json config 3): a
+discriminator Adam step on a batch of real and a batch of generated images, then one generator
+Adam step, through the operator graph and the HIP backend.  Inputs (z, images, labels) and all
+parameters are resident in HBM before the timed region starts; synthetic data, random-init weights.
+
+Prints ONE JSON line.  Besides the contract fields it carries
+  roofline      the dominant convolution kernel: algorithmic FLOP/s (HIP events around every launch
+                of that kernel inside the timed region) against the fp32 MFMA peak
+  cpu_baseline  the reference's own CPU operators (oracle/_ref, RT_MODE=CPU arithmetic) timed on this
+                host on a bounded sample and extrapolated to one iteration by FLOPs per operator class
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as ge  # noqa: E402
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_HBM_GBS = 8000.0
+
+# DCGAN layers: (H, W, C, O) of the equivalent forward convolution, 5x5, stride 2, SAME
+LAYERS = [(64, 64, 3, 64), (32, 32, 64, 128), (16, 16, 128, 256), (8, 8, 256, 512)]
+
+
+def conv_flops(batch, layer):
+    H, W, C, O = layer
+    return 2.0 * batch * (H // 2) * (W // 2) * O * 25 * C
+
+
+def iteration_flops(batch):
+    """Algorithmic FLOPs of one iteration by operator class (fwd-type, dx-type, dk-type convs and
+    the dense layers).  D step: G fwd, D fwd x2, dk x2, dx (layers 1-3) x2.  G step: G fwd, D fwd,
+    D dx (all layers), G dk, G dx (= fwd-type convs of layers 1-3)."""
+    f = [conv_flops(batch, l) for l in LAYERS]
+    all4, top3 = sum(f), sum(f[1:])
+    fwd = 2 * all4 + all4 + top3            # D fwd (2 + 1 times) + G input gradients
+    dx = all4 + 2 * top3 + all4 + all4      # G fwd (D step), D dx x2, G fwd (G step), D dx
+    dk = 2 * all4 + all4                    # D dk x2, G dk
+    dense = 2.0 * batch * (100 * 8192 + 8192) * 3 * 2
+    return {"fwd": fwd, "dx": dx, "dk": dk, "dense": dense, "total": fwd + dx + dk + dense}
+
+
+def synthetic(batch, seed=1234):
+    rng = np.random.default_rng(seed)
+    pkg = ge.load_package()
+    weights = {}
+    for name, shape in pkg.hostabi.var_shapes().items():
+        if name.endswith("_w"):
+            weights[name] = (rng.standard_normal(shape) * 0.02).astype(np.float32)
+        else:
+            weights[name] = np.zeros(shape, np.float32)
+    z = rng.uniform(-1, 1, (batch, 100)).astype(np.float32)
+    x = rng.uniform(-1, 1, (batch, 64, 64, 3)).astype(np.float32)
+    return weights, z, x
+
+
+def cpu_baseline(batch, budget_s=25.0):
+    """Times the reference's CPU operators (compiled from its own header into oracle/_ref) on one
+    core: conv2d, conv2d_input_grad, conv2d_kernel_grad on layer D1 at batch 1 (and D0 for the
+    cheap forward), then extrapolates one iteration from the measured FLOP/s of each class."""
+    oracle = ge.load_oracle()
+    kind = "reference" if oracle.have_ref() else "port"
+    orc = oracle.Oracle("ref" if kind == "reference" else "orc")
+    orc.set_threads(1)
+    rng = np.random.default_rng(0)
+    H, W, C, O = LAYERS[1]
+    n = 1
+    x = rng.uniform(-1, 1, (n, H, W, C)).astype(np.float32)
+    k = (rng.standard_normal((5, 5, C, O)) * 0.02).astype(np.float32)
+    dy = rng.uniform(-1, 1, (n, H // 2, W // 2, O)).astype(np.float32)
+    fl = conv_flops(n, LAYERS[1])
+    rates = {}
+    t0 = time.perf_counter()
+    orc.conv2d(x, k, (2, 2))
+    rates["fwd"] = fl / (time.perf_counter() - t0)
+    t0 = time.perf_counter()
+    orc.conv2d_input_grad(dy, k, 2, (H, W))
+    rates["dx"] = fl / (time.perf_counter() - t0)
+    t0 = time.perf_counter()
+    orc.conv2d_kernel_grad(dy, x, 2, (3, 3))
+    rates["dk"] = fl / (time.perf_counter() - t0)
+    work = iteration_flops(batch)
+    seconds = sum(work[c] / rates[c] for c in ("fwd", "dx", "dk")) + work["dense"] / rates["fwd"]
+    return {"value": 1.0 / seconds, "unit": "iterations/s", "cores": 1, "kind": kind,
+            "sample": "reference cpu::conv2d / conv2d_input_grad / conv2d_kernel_grad on layer D1 "
+                      "([1,32,32,64] -> 128, 5x5, s2) once each, one thread; iteration time extrapolated "
+                      "from the per-class GFLOP/s (%.3f / %.3f / %.3f) over %.0f GFLOP"
+                      % (rates["fwd"] / 1e9, rates["dx"] / 1e9, rates["dk"] / 1e9, work["total"] / 1e9),
+            "gflops": {c: rates[c] / 1e9 for c in rates}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--fusion", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
+
+    pkg = ge.load_package()
+    A = pkg.hipabi
+    weights, z, x = synthetic(args.batch)
+    model = pkg.hostabi.DcganModel(args.batch, seed=1, mode="GPU")
+    model.set_fusion(bool(args.fusion))
+    for name, w in weights.items():
+        model.set_var(name, w)
+    model.set_inputs(z, x)   # resident from here on
+
+    def iteration():
+        model.d_step(want_loss=False)
+        model.g_step(want_loss=False)
+
+    for _ in range(args.warmup):
+        iteration()
+    model.sync()
+
+    A.profile_reset()
+    A.profile_enable(True)
+    timer = A.Timer()           # events on the stream the kernels run on (the default stream)
+    t0 = time.perf_counter()
+    timer.start()
+    for _ in range(args.steps):
+        iteration()
+    gpu_ms = timer.stop_ms()    # waits for the stop event
+    model.sync()
+    wall = time.perf_counter() - t0
+    A.profile_enable(False)
+    rows = A.profile_read()
+    d_loss = model.eval("d_loss")[0]
+    g_loss = model.eval("g_loss")[0]
+
+    ms_per_step = wall * 1e3 / args.steps
+    work = iteration_flops(args.batch)
+    conv_ms = sum(r["ms"] for r in rows)
+    conv_fl = sum(r["flops"] for r in rows)
+    dom = max(rows, key=lambda r: r["ms"])
+    achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+    roofline = {
+        "kernel": dom["name"], "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "launches": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 2),
+        "flops_per_launch": dom["flops"] / dom["launches"],
+        "all_conv_kernels": {"tflops": round(conv_fl / (conv_ms * 1e-3) / 1e12, 3),
+                             "frac": round(conv_fl / (conv_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                             "ms_per_step": round(conv_ms / args.steps, 4)},
+        "kernels": [{"name": r["name"], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+                     "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2)} for r in sorted(rows, key=lambda r: -r["ms"])],
+    }
+    out = {
+        "metric": "DCGAN train iters/sec @bs64 fp32; conv(_transpose) TFLOP/s as % fp32-MFMA peak",
+        "value": round(args.steps / wall, 3), "unit": "iterations/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[3]: full DCGAN training iteration (D step on real+fake, one G step, Adam), "
+                               "fp32, batch %d, 64x64x3 images, z dim 100" % args.batch,
+                   "batch": args.batch, "fusion": bool(args.fusion)},
+        "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
+        "iteration_gflop": round(work["total"] / 1e9, 2),
+        "iteration_tflops": round(work["total"] / (wall / args.steps) / 1e12, 3),
+        "losses_after": {"d_loss": float(d_loss), "g_loss": float(g_loss)},
+        "device": A.device_info(),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.batch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -8,3 +8,4 @@ importlib) under the module name `dcgan_cuda_amd`.
 """
 from . import hipabi  # noqa: F401
 from .hipabi import Buf, HipBackend, load  # noqa: F401
+from . import hostabi  # noqa: F401

@@ -17,6 +17,10 @@
 // im2col + GEMM + re-layout pipeline this replaces).
 #include "dh_common.h"
 
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
 using namespace dh;
 
 namespace
@@ -452,9 +456,66 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ p
 
 struct TileCfg { int bm, bn; };
 
+// Optional per-kernel timing: when enabled, every conv_igemm launch is bracketed by two HIP events
+// on its stream and tagged with the kernel instantiation and the algorithmic FLOPs of the operator
+// it belongs to.  dh_profile_read() waits for the events and adds them up per tag.
+struct ProfRecord
+{
+    hipEvent_t e0, e1;
+    int tag;
+    double flops;
+};
+struct ProfTotal
+{
+    char name[96];
+    long launches;
+    double ms, flops;
+};
+bool g_prof_on = false;
+std::vector<ProfRecord> g_prof_pending;
+std::vector<hipEvent_t> g_prof_pool;
+std::vector<ProfTotal> g_prof_totals;
+double g_prof_flops = 0.0;  // algorithmic FLOPs of the operator being launched
+
+int prof_tag(const char* name)
+{
+    for (size_t i = 0; i < g_prof_totals.size(); ++i)
+        if (!strcmp(g_prof_totals[i].name, name))
+            return (int)i;
+    ProfTotal t{};
+    snprintf(t.name, sizeof(t.name), "%s", name);
+    g_prof_totals.push_back(t);
+    return (int)g_prof_totals.size() - 1;
+}
+
+hipEvent_t prof_event()
+{
+    if (!g_prof_pool.empty())
+    {
+        hipEvent_t e = g_prof_pool.back();
+        g_prof_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+
 template <int MODE, int BM, int BN, int WGM, int WGN>
 int launch_cfg(const ConvParams& p, dim3 grid, bool veca, bool vecb, hipStream_t st)
 {
+    ProfRecord rec{};
+    if (g_prof_on)
+    {
+        char name[96];
+        snprintf(name, sizeof(name), "conv_igemm<%s,%dx%d,%s%s>", MODE == MODE_FWD ? "fwd" : MODE == MODE_DX ? "dx" : "dk",
+                 BM, BN, veca ? "v" : "s", vecb ? "v" : "s");
+        rec.tag = prof_tag(name);
+        rec.flops = g_prof_flops;
+        rec.e0 = prof_event();
+        rec.e1 = prof_event();
+        (void)hipEventRecord(rec.e0, st);
+    }
     if (veca && vecb)
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, true, true>), grid, dim3(NTHREADS), 0, st, p);
     else if (veca)
@@ -463,6 +524,11 @@ int launch_cfg(const ConvParams& p, dim3 grid, bool veca, bool vecb, hipStream_t
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, false, true>), grid, dim3(NTHREADS), 0, st, p);
     else
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, false, false>), grid, dim3(NTHREADS), 0, st, p);
+    if (g_prof_on)
+    {
+        (void)hipEventRecord(rec.e1, st);
+        g_prof_pending.push_back(rec);
+    }
     DH_LAUNCH_CHECK("conv_igemm launch");
     return 0;
 }
@@ -581,6 +647,7 @@ int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W,
     }
     const bool veca = C % 4 == 0 && aligned16(x);
     const bool vecb = O % 4 == 0 && aligned16(k);
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C;
     DH_TRY(run_igemm<MODE_FWD>(p, 1, p.phase[0].M, veca, vecb, as_stream(stream), cfg));
     return finish_splitk(p, as_stream(stream));
 }
@@ -638,6 +705,8 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
     }
     const bool veca = O % 4 == 0 && aligned16(dy);
     const bool vecb = O % 4 == 0 && aligned16(k);
+    // one launch covers up to MAX_PHASES phases; the operator's FLOPs are split evenly over launches
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C / ((n_live + MAX_PHASES - 1) / MAX_PHASES > 0 ? (n_live + MAX_PHASES - 1) / MAX_PHASES : 1);
     for (int z0 = 0; z0 < n_live; z0 += MAX_PHASES)
     {
         const int nz = n_live - z0 < MAX_PHASES ? n_live - z0 : MAX_PHASES;
@@ -676,8 +745,62 @@ int dh_conv2d_dk(const float* x, const float* dy, float* dk, int N, int H, int W
     }
     const bool veca = C % 4 == 0 && aligned16(x);
     const bool vecb = O % 4 == 0 && aligned16(dy);
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C;
     DH_TRY(run_igemm<MODE_DK>(p, 1, p.phase[0].M, veca, vecb, as_stream(stream), cfg));
     return finish_splitk(p, as_stream(stream));
+}
+
+
+int dh_profile_enable(int on)
+{
+    DH_TRY(ensure_init());
+    g_prof_on = on != 0;
+    return 0;
+}
+
+int dh_profile_reset(void)
+{
+    DH_TRY(ensure_init());
+    DH_HIP(hipDeviceSynchronize());
+    for (ProfRecord& r : g_prof_pending)
+    {
+        g_prof_pool.push_back(r.e0);
+        g_prof_pool.push_back(r.e1);
+    }
+    g_prof_pending.clear();
+    g_prof_totals.clear();
+    return 0;
+}
+
+int dh_profile_read(char* buf, size_t buf_len)
+{
+    DH_TRY(ensure_init());
+    for (ProfRecord& r : g_prof_pending)
+    {
+        float ms = 0.f;
+        DH_HIP(hipEventSynchronize(r.e1));
+        DH_HIP(hipEventElapsedTime(&ms, r.e0, r.e1));
+        ProfTotal& t = g_prof_totals[r.tag];
+        t.launches += 1;
+        t.ms += ms;
+        t.flops += r.flops;
+        g_prof_pool.push_back(r.e0);
+        g_prof_pool.push_back(r.e1);
+    }
+    g_prof_pending.clear();
+    size_t used = 0;
+    if (buf && buf_len)
+        buf[0] = 0;
+    for (const ProfTotal& t : g_prof_totals)
+    {
+        if (!buf || used >= buf_len)
+            break;
+        const int w = snprintf(buf + used, buf_len - used, "%s\t%ld\t%.6f\t%.0f\n", t.name, t.launches, t.ms, t.flops);
+        if (w < 0 || (size_t)w >= buf_len - used)
+            return fail(DH_EINVAL, "dh_profile_read: buffer too small");
+        used += (size_t)w;
+    }
+    return 0;
 }
 
 }

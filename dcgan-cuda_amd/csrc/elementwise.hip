@@ -581,16 +581,15 @@ int dh_adam_update(float* p, const float* m, const float* v, float lrt, float ep
     return 0;
 }
 
-int dh_adam_step(float* p, float* m, float* v, const float* g, float beta1, float beta2, float lrt, float eps,
-                 size_t n, void* stream)
+int dh_adam_step(float* p, float* m, float* v, const float* g, float m_decay, float m_gain, float v_decay,
+                 float v_gain, float lrt, float eps, size_t n, void* stream)
 {
     DH_TRY(ensure_init());
     if (n == 0) return 0;
     if (!p || !m || !v || !g) return fail(DH_EINVAL, "dh_adam_step: null tensor");
     const bool vec = aligned16(p) && aligned16(m) && aligned16(v) && aligned16(g);
-    // 1 - beta in float, as src/api/adam-optimizer.cu forms the second coefficient
     hipLaunchKernelGGL(adam_step_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), p, m, v, g,
-                       beta1, 1.f - beta1, beta2, 1.f - beta2, lrt, eps, n, vec);
+                       m_decay, m_gain, v_decay, v_gain, lrt, eps, n, vec);
     DH_LAUNCH_CHECK("dh_adam_step");
     return 0;
 }

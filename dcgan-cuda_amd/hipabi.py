@@ -37,6 +37,9 @@ _SIGS = {
     "dh_event_record": [_vp, _vp],
     "dh_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "dh_workspace_reserve": [_sz],
+    "dh_profile_enable": [_i],
+    "dh_profile_reset": [],
+    "dh_profile_read": [C.c_char_p, _sz],
     "dh_conv2d_fwd": [_vp, _vp, _vp] + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dx": [_vp, _vp, _vp] + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dk": [_vp, _vp, _vp] + [_i] * 13 + [_vp],
@@ -64,7 +67,7 @@ _SIGS = {
     "dh_moment_update": [_vp, _vp, _f, _f, _sz, _vp],
     "dh_moment_update2": [_vp, _vp, _f, _f, _sz, _vp],
     "dh_adam_update": [_vp, _vp, _vp, _f, _f, _sz, _vp],
-    "dh_adam_step": [_vp, _vp, _vp, _vp, _f, _f, _f, _f, _sz, _vp],
+    "dh_adam_step": [_vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _f, _sz, _vp],
     "dh_sgd_update": [_vp, _vp, _vp, _sz, _vp],
 }
 _RESTYPES = {"dh_version": C.c_char_p, "dh_last_error": C.c_char_p, "dh_workspace_bytes": _sz}
@@ -175,6 +178,25 @@ class Timer:
         ms = _f()
         check(load().dh_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
         return ms.value
+
+
+def profile_enable(on):
+    check(load().dh_profile_enable(1 if on else 0))
+
+
+def profile_reset():
+    check(load().dh_profile_reset())
+
+
+def profile_read():
+    """[{name, launches, ms, flops}] per convolution-kernel instantiation since the last reset."""
+    buf = C.create_string_buffer(1 << 16)
+    check(load().dh_profile_read(buf, len(buf)))
+    rows = []
+    for line in buf.value.decode().splitlines():
+        name, n, ms, fl = line.split("\t")
+        rows.append({"name": name, "launches": int(n), "ms": float(ms), "flops": float(fl)})
+    return rows
 
 
 def same_pad(n_in, k, s):
@@ -408,7 +430,9 @@ class HipBackend:
 
     def adam_step(self, p, m, v, g, beta1, beta2, lrt, eps):
         dp, dm, dv, dg = self._up(p, m, v, g)
-        check(self.lib.dh_adam_step(dp.ptr, dm.ptr, dv.ptr, dg.ptr, beta1, beta2, lrt, eps, dp.size, self.stream))
+        one = np.float32(1)
+        check(self.lib.dh_adam_step(dp.ptr, dm.ptr, dv.ptr, dg.ptr, beta1, one - np.float32(beta1), beta2,
+                                    one - np.float32(beta2), lrt, eps, dp.size, self.stream))
         return dp.numpy(), dm.numpy(), dv.numpy()
 
     def vect_update(self, var, dv, coeff):

@@ -1,0 +1,352 @@
+#include "dcgan.hh"
+
+#include <cstring>
+#include <stdexcept>
+
+#include "backend.hh"
+#include "memory.hh"
+
+namespace dcgan
+{
+
+namespace
+{
+constexpr int Z_DIM = 100;
+int g_strides[2] = {2, 2};
+
+ops::Op* transpose_block(ops::Op* input, const int* in_size, const int* out_size, bool use_activ,
+                         Conv2DTransposeLayerData& data, Initializer& w_init)
+{
+    auto& builder = ops::OpsBuilder::instance();
+    auto w = builder.variable(ops::Shape({5, 5, out_size[3], in_size[3]}), true);
+    w->extend_name("conv2d_transpose_w");
+    auto b = builder.variable(ops::Shape({out_size[3]}), true);
+    b->extend_name("conv2d_transpose_b");
+    ZeroInitializer zero;
+    w_init.fill(w->data_begin(), w->data_end());
+    zero.fill(b->data_begin(), b->data_end());
+    ops::Op* z = builder.conv2d_bias_add(builder.conv2d_transpose(input, w, out_size, g_strides), b);
+    data = {w, b, z};
+    if (!use_activ)
+        return z;
+    ops::Op* out = relu(z);
+    out->extend_name("conv2d_transpose_activ");
+    return out;
+}
+
+ops::Op* conv_block(ops::Op* input, int in_channels, int nb_filter, Conv2DLayerData& data, bool reuse,
+                    Initializer& w_init)
+{
+    auto& builder = ops::OpsBuilder::instance();
+    if (!reuse)
+    {
+        auto w = builder.variable(ops::Shape({5, 5, in_channels, nb_filter}), true);
+        w->extend_name("conv2d_w");
+        auto b = builder.variable(ops::Shape({nb_filter}), true);
+        b->extend_name("conv2d_b");
+        ZeroInitializer zero;
+        w_init.fill(w->data_begin(), w->data_end());
+        zero.fill(b->data_begin(), b->data_end());
+        data.w = w;
+        data.b = b;
+    }
+    ops::Op* z = builder.conv2d_bias_add(builder.conv2d(input, data.w, g_strides), data.b);
+    data.z = z;
+    ops::Op* out = leaky_relu(z);
+    out->extend_name("conv2d_activ");
+    return out;
+}
+
+ops::Op* discriminator(Model& m, ops::Op* x, std::vector<ops::Op*>& nodes, Initializer& w_init)
+{
+    auto& builder = ops::OpsBuilder::instance();
+    const bool reuse = !m.d_layers.empty();
+    if (!reuse)
+        m.d_layers.resize(4);
+    const int chans[5] = {3, 64, 128, 256, 512};
+    ops::Op* cur = x;
+    for (int l = 0; l < 4; ++l)
+    {
+        cur = conv_block(cur, chans[l], chans[l + 1], m.d_layers[l], reuse, w_init);
+        nodes.push_back(cur);
+    }
+    cur = builder.reshape(cur, ops::Shape({m.batch, 4 * 4 * 512}));
+    if (!reuse)
+    {
+        auto w = builder.variable(ops::Shape({4 * 4 * 512, 1}), true);
+        w->extend_name("dense_w");
+        auto b = builder.variable(ops::Shape({1}), true);
+        b->extend_name("dense_b");
+        ZeroInitializer zero;
+        w_init.fill(w->data_begin(), w->data_end());
+        zero.fill(b->data_begin(), b->data_end());
+        m.d_dense.w = w;
+        m.d_dense.b = b;
+    }
+    ops::Op* logits = builder.mat_mul_add(cur, m.d_dense.w, m.d_dense.b);
+    m.d_dense.z = logits;
+    nodes.push_back(logits);
+    return logits;
+}
+}  // namespace
+
+Model* build(int batch, unsigned long long seed)
+{
+    auto& builder = ops::OpsBuilder::instance();
+    auto* mp = new Model;
+    Model& m = *mp;
+    m.batch = batch;
+    NormalInitializer w_init(0, 0.02, seed);
+
+    m.z = builder.input(ops::Shape({batch, Z_DIM}));
+    m.x = builder.input(ops::Shape({batch, 64, 64, 3}));
+
+    // generator (dcgan/main.cu:89-120)
+    ZeroInitializer zero;
+    ops::Op* l0 = dense_layer(m.z, Z_DIM, 4 * 4 * 512, relu, &w_init, &zero, &m.g_dense);
+    l0 = builder.reshape(l0, ops::Shape({batch, 4, 4, 512}));
+    m.g_nodes.push_back(l0);
+    const int sizes[5][4] = {{batch, 4, 4, 512}, {batch, 8, 8, 256}, {batch, 16, 16, 128}, {batch, 32, 32, 64},
+                             {batch, 64, 64, 3}};
+    m.g_layers.resize(4);
+    ops::Op* cur = l0;
+    for (int l = 0; l < 4; ++l)
+    {
+        cur = transpose_block(cur, sizes[l], sizes[l + 1], l < 3, m.g_layers[l], w_init);
+        m.g_nodes.push_back(cur);
+    }
+    m.g_out = builder.vect_tanh(cur);
+
+    // discriminator on generated and on real images, shared weights (dcgan/main.cu:217-249, :293-297)
+    ops::Op* fake_logits = discriminator(m, m.g_out, m.d_fake_nodes, w_init);
+    ops::Op* real_logits = discriminator(m, m.x, m.d_real_nodes, w_init);
+
+    m.labels0 = builder.input(ops::Shape({batch, 1}));
+    m.labels1 = builder.input(ops::Shape({batch, 1}));
+    m.zeros.assign(batch, 0.f);
+    m.ones.assign(batch, 1.f);
+
+    // losses (dcgan/main.cu:304-307)
+    m.g_loss = builder.sigmoid_cross_entropy(m.labels1, fake_logits);
+    m.d_fake_loss = builder.sigmoid_cross_entropy(m.labels0, fake_logits);
+    m.d_real_loss = builder.sigmoid_cross_entropy(m.labels1, real_logits);
+    m.d_loss = builder.add(m.d_fake_loss, m.d_real_loss);
+
+    for (auto& l : m.g_layers)
+    {
+        m.g_vars.push_back(dynamic_cast<ops::Variable*>(l.w));
+        m.g_vars.push_back(dynamic_cast<ops::Variable*>(l.b));
+    }
+    m.g_vars.push_back(dynamic_cast<ops::Variable*>(m.g_dense.w));
+    m.g_vars.push_back(dynamic_cast<ops::Variable*>(m.g_dense.b));
+    for (auto& l : m.d_layers)
+    {
+        m.d_vars.push_back(dynamic_cast<ops::Variable*>(l.w));
+        m.d_vars.push_back(dynamic_cast<ops::Variable*>(l.b));
+    }
+    m.d_vars.push_back(dynamic_cast<ops::Variable*>(m.d_dense.w));
+    m.d_vars.push_back(dynamic_cast<ops::Variable*>(m.d_dense.b));
+
+    // Adam(2e-4, 0.5) for each network (dcgan/main.cu:329-332)
+    AdamOptimizer g_adam(0.0002, 0.5);
+    m.g_opti = g_adam.minimize(m.g_loss, m.g_vars);
+    AdamOptimizer d_adam(0.0002, 0.5);
+    m.d_opti = d_adam.minimize(m.d_loss, m.d_vars);
+    return mp;
+}
+
+}  // namespace dcgan
+
+namespace
+{
+thread_local std::string g_error;
+
+template <class F>
+int guarded(F f)
+{
+    try
+    {
+        f();
+        return 0;
+    }
+    catch (const std::exception& e)
+    {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+dcgan::Model& M(void* p) { return *static_cast<dcgan::Model*>(p); }
+
+ops::Variable* var_at(dcgan::Model& m, int i)
+{
+    const int ng = (int)m.g_vars.size();
+    if (i < 0 || i >= ng + (int)m.d_vars.size())
+        throw std::runtime_error("variable index out of range");
+    return i < ng ? m.g_vars[i] : m.d_vars[i - ng];
+}
+
+void bind_labels(dcgan::Model& m)
+{
+    // the label inputs are constants: bound once, then resident
+    auto& g = ops::Graph::instance();
+    const ops::Shape s({m.batch, 1});
+    g.run({m.labels0, m.labels1}, {{m.labels0, {m.zeros.data(), s}}, {m.labels1, {m.ones.data(), s}}}, {});
+}
+
+ops::Op* lookup(dcgan::Model& m, const std::string& what)
+{
+    auto& g = ops::Graph::instance();
+    auto layer = [&](const std::string& prefix, std::vector<ops::Op*>& nodes, const char* last) -> ops::Op* {
+        if (what == prefix + last)
+            return nodes.back();
+        for (std::size_t i = 0; i + 1 < nodes.size() || (i < nodes.size() && !*last); ++i)
+            if (what == prefix + "l" + std::to_string(i))
+                return nodes[i];
+        return nullptr;
+    };
+    if (what == "g_out") return m.g_out;
+    if (what == "g_loss") return m.g_loss;
+    if (what == "d_loss") return m.d_loss;
+    if (what == "d_fake_loss") return m.d_fake_loss;
+    if (what == "d_real_loss") return m.d_real_loss;
+    if (what.rfind("g_l", 0) == 0)
+    {
+        const int i = std::stoi(what.substr(3));
+        return m.g_nodes.at(i);
+    }
+    if (ops::Op* o = layer("d_fake_", m.d_fake_nodes, "logits")) return o;
+    if (ops::Op* o = layer("d_real_", m.d_real_nodes, "logits")) return o;
+    if (what.rfind("grad:", 0) == 0)
+    {
+        const std::size_t c = what.find(':', 5);
+        const std::string loss = what.substr(5, c - 5), target = what.substr(c + 1);
+        ops::Op* l = loss == "g_loss" ? m.g_loss : loss == "d_loss" ? m.d_loss : nullptr;
+        if (!l)
+            throw std::runtime_error("unknown loss " + loss);
+        if (target == "x_fake")
+            return g.gradient(l, m.g_out);
+        return g.gradient(l, var_at(m, std::stoi(target)));
+    }
+    throw std::runtime_error("unknown tensor " + what);
+}
+}  // namespace
+
+extern "C" {
+
+const char* dg_last_error(void) { return g_error.c_str(); }
+
+void* dg_create(int batch, unsigned long long seed)
+{
+    dcgan::Model* m = nullptr;
+    if (guarded([&] {
+            m = dcgan::build(batch, seed);
+            bind_labels(*m);
+        }))
+        return nullptr;
+    return m;
+}
+
+void dg_destroy(void* model)
+{
+    guarded([&] {
+        ops::Graph::instance().exit_graph();
+        delete static_cast<dcgan::Model*>(model);
+    });
+}
+
+void dg_set_fusion(int fuse)
+{
+    hip::set_fusion(fuse != 0);
+    hip::forget_plans();
+}
+
+int dg_num_vars(void* model) { return (int)(M(model).g_vars.size() + M(model).d_vars.size()); }
+
+long dg_var_size(void* model, int index)
+{
+    long n = -1;
+    guarded([&] { n = var_at(M(model), index)->shape_get().total(); });
+    return n;
+}
+
+int dg_var_read(void* model, int index, float* host)
+{
+    return guarded([&] { var_at(M(model), index)->read(host); });
+}
+
+int dg_var_write(void* model, int index, const float* host)
+{
+    return guarded([&] { var_at(M(model), index)->write(host); });
+}
+
+int dg_set_inputs(void* model, const float* z_host, const float* x_host)
+{
+    return guarded([&] {
+        dcgan::Model& m = M(model);
+        std::map<ops::Input*, std::pair<const dbl_t*, ops::Shape>> in;
+        std::vector<ops::Op*> targets;
+        if (z_host)
+        {
+            in[m.z] = {z_host, ops::Shape({m.batch, 100})};
+            targets.push_back(m.z);
+        }
+        if (x_host)
+        {
+            in[m.x] = {x_host, ops::Shape({m.batch, 64, 64, 3})};
+            targets.push_back(m.x);
+        }
+        ops::Graph::instance().run(targets, in, {});
+    });
+}
+
+int dg_d_step(void* model, float* d_loss)
+{
+    return guarded([&] {
+        dcgan::Model& m = M(model);
+        hip::set_sync_each_run(d_loss != nullptr);
+        ops::Graph::instance().run({m.d_opti, m.d_loss}, {}, {nullptr, d_loss});
+        hip::set_sync_each_run(true);
+    });
+}
+
+int dg_g_step(void* model, float* g_loss)
+{
+    return guarded([&] {
+        dcgan::Model& m = M(model);
+        hip::set_sync_each_run(g_loss != nullptr);
+        ops::Graph::instance().run({m.g_opti, m.g_loss}, {}, {nullptr, g_loss});
+        hip::set_sync_each_run(true);
+    });
+}
+
+int dg_sync(void)
+{
+    return guarded([] {
+        if (program_mode() == ProgramMode::GPU)
+            hip::synchronize();
+    });
+}
+
+int dg_generate(void* model, float* images_host)
+{
+    return guarded([&] { ops::Graph::instance().run({M(model).g_out}, {}, {images_host}); });
+}
+
+int dg_eval(void* model, const char* what, float* host, long* count)
+{
+    return guarded([&] {
+        ops::Op* op = lookup(M(model), what);
+        if (count)
+            *count = op->shape_get().total();
+        if (host)
+            ops::Graph::instance().run({op}, {}, {host});
+    });
+}
+
+int dg_last_schedule_size(void*)
+{
+    return (int)ops::Graph::instance().last_schedule().size();
+}
+
+}

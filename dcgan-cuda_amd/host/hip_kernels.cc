@@ -1,0 +1,630 @@
+// The HIP backend seen from the operator graph: a kernel table indexed by rt::Node::type and a
+// runner, i.e. the drop-in for gpu::kernels_list / gpu::run (src/gpu/kernels.cu:23-61,
+// src/gpu/runner.cu:10-18).  Each table entry decodes the node exactly as the reference's GPU
+// entry does (citations per function) and makes one C-ABI call; nothing else happens here.
+#include "backend.hh"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "dcgan_hip.h"
+#include "memory.hh"
+
+namespace hip
+{
+
+namespace
+{
+
+void* g_stream = nullptr;  // the default stream; every launch of the backend is ordered on it
+int g_fusion = -1;         // -1: not decided yet (reads DCGAN_HIP_FUSE)
+
+#define CK(call) hip_check((call), #call)
+
+struct ConvGeom
+{
+    int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
+};
+
+// conv2d forward.  Node fields: src/runtime/node.cu:118-141; decode: src/gpu/conv2d.cu:13-40.
+ConvGeom geom_conv2d(const rt::Node* n)
+{
+    ConvGeom g;
+    g.N = n->sizes1[0]; g.H = n->sizes1[1]; g.W = n->sizes1[2]; g.C = n->sizes1[3];
+    g.kh = n->sizes2[0]; g.kw = n->sizes2[1]; g.O = n->sizes2[3];
+    g.sh = n->intconst[0]; g.sw = n->intconst[1];
+    const int pad_h = n->int_cons1, pad_w = n->int_cons2;  // totals; the part before is half, rounded down
+    g.pt = pad_h / 2; g.pl = pad_w / 2;
+    g.Ho = (g.H + pad_h - g.kh) / g.sh + 1;
+    g.Wo = (g.W + pad_w - g.kw) / g.sw + 1;
+    return g;
+}
+
+// conv2d input gradient.  Fields: src/runtime/node.cu:171-193; decode: src/gpu/conv2d.cu:70-98
+// (one stride for both axes, pads re-derived from the extents).
+ConvGeom geom_input_grad(const rt::Node* n)
+{
+    ConvGeom g;
+    g.N = n->sizes1[0]; g.Ho = n->sizes1[1]; g.Wo = n->sizes1[2]; g.O = n->sizes1[3];
+    g.kh = n->sizes2[0]; g.kw = n->sizes2[1]; g.C = n->sizes2[2];
+    g.sh = g.sw = n->intconst[0];
+    g.H = n->intconst2[0]; g.W = n->intconst2[1];
+    g.pt = ((g.Ho - 1) * g.sh - g.H + g.kh) / 2;
+    g.pl = ((g.Wo - 1) * g.sw - g.W + g.kw) / 2;
+    return g;
+}
+
+// conv2d filter gradient.  Fields: src/runtime/node.cu:195-217; decode: src/gpu/conv2d.cu:119-146
+// (filter extent derived as H + pad - s*(Ho-1)).
+ConvGeom geom_kernel_grad(const rt::Node* n)
+{
+    ConvGeom g;
+    g.N = n->sizes2[0]; g.H = n->sizes2[1]; g.W = n->sizes2[2]; g.C = n->sizes2[3];
+    g.Ho = n->sizes1[1]; g.Wo = n->sizes1[2]; g.O = n->sizes1[3];
+    g.sh = n->intconst[0]; g.sw = n->intconst[1];
+    const int pad_h = n->intconst2[0], pad_w = n->intconst2[1];
+    g.pt = pad_h / 2; g.pl = pad_w / 2;
+    g.kh = g.H + pad_h - g.sh * (g.Ho - 1);
+    g.kw = g.W + pad_w - g.sw * (g.Wo - 1);
+    return g;
+}
+
+// conv2d_transpose forward = input gradient of the conv whose "y" is this op's input.
+// Fields: src/runtime/node.cu:219-243; decode: src/gpu/conv2d.cu:167-196.
+ConvGeom geom_transpose(const rt::Node* n)
+{
+    ConvGeom g;
+    g.N = n->sizes2[0]; g.Ho = n->sizes2[1]; g.Wo = n->sizes2[2]; g.O = n->sizes2[3];
+    g.kh = n->sizes3[0]; g.kw = n->sizes3[1]; g.C = n->sizes3[2];
+    g.sh = n->intconst[0]; g.sw = n->intconst[1];
+    g.H = n->sizes1[1]; g.W = n->sizes1[2];
+    g.pt = ((g.Ho - 1) * g.sh - g.H + g.kh) / 2;
+    g.pl = ((g.Wo - 1) * g.sw - g.W + g.kw) / 2;
+    return g;
+}
+
+// conv2d_transpose input gradient = forward conv of dy.  Fields: src/runtime/node.cu:245-267;
+// decode: src/gpu/conv2d.cu:214-241.
+ConvGeom geom_transpose_input_grad(const rt::Node* n)
+{
+    ConvGeom g;
+    g.N = n->sizes1[0]; g.H = n->sizes1[1]; g.W = n->sizes1[2]; g.C = n->sizes2[2];
+    g.kh = n->sizes2[0]; g.kw = n->sizes2[1]; g.O = n->sizes2[3];
+    g.sh = g.sw = n->intconst[0];
+    g.Ho = n->intconst2[0]; g.Wo = n->intconst2[1];
+    g.pt = ((g.Ho - 1) * g.sh + g.kh - g.H) / 2;
+    g.pl = ((g.Wo - 1) * g.sw + g.kw - g.W) / 2;
+    return g;
+}
+
+// conv2d_transpose filter gradient = conv2d filter gradient with dy in the role of the image and
+// the transpose's input in the role of the output gradient.  Fields: src/runtime/node.cu:269-294;
+// decode: src/gpu/conv2d.cu:264-289.
+ConvGeom geom_transpose_kernel_grad(const rt::Node* n)
+{
+    ConvGeom g;
+    g.N = n->sizes2[0]; g.Ho = n->sizes2[1]; g.Wo = n->sizes2[2]; g.O = n->sizes2[3];  // transpose input
+    g.H = n->sizes1[1]; g.W = n->sizes1[2]; g.C = n->sizes1[3];                        // dy
+    g.kh = n->sizes3[0]; g.kw = n->sizes3[1];
+    g.sh = n->intconst[0]; g.sw = n->intconst[1];
+    g.pt = ((g.Ho - 1) * g.sh + g.kh - g.H) / 2;
+    g.pl = ((g.Wo - 1) * g.sw + g.kw - g.W) / 2;
+    return g;
+}
+
+void conv_fwd(const ConvGeom& g, const dbl_t* x, const dbl_t* k, dbl_t* y, const dbl_t* bias, int act, float alpha)
+{
+    CK(dh_conv2d_fwd(x, k, y, g.N, g.H, g.W, g.C, g.kh, g.kw, g.O, g.sh, g.sw, g.pt, g.pl, g.Ho, g.Wo, bias, act,
+                     alpha, g_stream));
+}
+
+void conv_dx(const ConvGeom& g, const dbl_t* dy, const dbl_t* k, dbl_t* dx, const dbl_t* bias, int act, float alpha)
+{
+    CK(dh_conv2d_dx(dy, k, dx, g.N, g.Ho, g.Wo, g.O, g.kh, g.kw, g.C, g.sh, g.sw, g.pt, g.pl, g.H, g.W, bias, act,
+                    alpha, g_stream));
+}
+
+void conv_dk(const ConvGeom& g, const dbl_t* x, const dbl_t* dy, dbl_t* dk)
+{
+    CK(dh_conv2d_dk(x, dy, dk, g.N, g.H, g.W, g.C, g.Ho, g.Wo, g.O, g.kh, g.kw, g.sh, g.sw, g.pt, g.pl, g_stream));
+}
+
+// ---- table entries -----------------------------------------------------------------------------
+void k_conv2d(rt::Node* n) { conv_fwd(geom_conv2d(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f); }
+void k_conv2d_input_grad(rt::Node* n) { conv_dx(geom_input_grad(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f); }
+void k_conv2d_kernel_grad(rt::Node* n) { conv_dk(geom_kernel_grad(n), n->in2, n->in1, n->out1); }
+void k_conv2d_transpose(rt::Node* n) { conv_dx(geom_transpose(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f); }
+void k_conv2d_transpose_input_grad(rt::Node* n)
+{
+    conv_fwd(geom_transpose_input_grad(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f);
+}
+void k_conv2d_transpose_kernel_grad(rt::Node* n) { conv_dk(geom_transpose_kernel_grad(n), n->in1, n->in2, n->out1); }
+
+// src/gpu/matmul.cu:88-150 (matmul, mvrow_add, matmul_add, tmat_mat_mul, mat_tmat_mul hosts)
+void k_mat_mat_mul(rt::Node* n) { CK(dh_gemm_nn(n->in1, n->in2, nullptr, n->out1, n->len1, n->len2, n->len3, g_stream)); }
+void k_mat_rvect_add(rt::Node* n) { CK(dh_bias_add(n->in1, n->in2, n->out1, n->len1, n->len2, g_stream)); }
+void k_mat_mul_add(rt::Node* n) { CK(dh_gemm_nn(n->in1, n->in2, n->in3, n->out1, n->len1, n->len2, n->len3, g_stream)); }
+void k_tmat_mat_mul(rt::Node* n) { CK(dh_gemm_tn(n->in1, n->in2, n->out1, n->len1, n->len2, n->len3, g_stream)); }
+void k_mat_tmat_mul(rt::Node* n) { CK(dh_gemm_nt(n->in1, n->in2, n->out1, n->len1, n->len2, n->len3, g_stream)); }
+// src/gpu/sum.cu:216-243
+void k_mat_sum_rows(rt::Node* n) { CK(dh_mat_sum_rows(n->in1, n->out1, n->len1, n->len2, g_stream)); }
+void k_mat_sum_cols(rt::Node* n) { CK(dh_bias_grad(n->in1, n->out1, n->len1, n->len2, g_stream)); }
+void k_mse(rt::Node* n) { CK(dh_mse(n->in1, n->in2, n->out1, n->len1, n->len2, g_stream)); }
+void k_mse_grad(rt::Node* n) { CK(dh_mse_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
+void k_argmax_acc(rt::Node* n) { CK(dh_argmax_acc(n->in1, n->in2, n->out1, n->len1, n->len2, g_stream)); }
+void k_add(rt::Node* n) { CK(dh_add(n->in1, n->in2, n->out1, n->len1, g_stream)); }
+// src/gpu/relu.cu:68-104
+void k_relu(rt::Node* n) { CK(dh_relu(n->in1, n->out1, n->len1, g_stream)); }
+void k_relu_leaky(rt::Node* n) { CK(dh_relu_leaky(n->in1, n->out1, n->len1, n->alpha_leaky, g_stream)); }
+void k_relu_grad(rt::Node* n) { CK(dh_relu_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
+void k_leaky_relu_grad(rt::Node* n) { CK(dh_leaky_relu_grad(n->in1, n->in2, n->out1, n->cons1, n->len1, g_stream)); }
+// src/gpu/sigmoid.cu:124-180
+void k_sigmoid(rt::Node* n) { CK(dh_sigmoid(n->in1, n->out1, n->len1, g_stream)); }
+void k_tanh(rt::Node* n) { CK(dh_tanh(n->in1, n->out1, n->len1, g_stream)); }
+void k_sigmoid_grad(rt::Node* n) { CK(dh_sigmoid_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
+void k_tanh_grad(rt::Node* n) { CK(dh_tanh_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
+void k_sigmoid_cross_entropy(rt::Node* n) { CK(dh_sigmoid_cross_entropy(n->in1, n->in2, n->out1, n->len1, g_stream)); }
+void k_sigmoid_cross_entropy_grad(rt::Node* n)
+{
+    CK(dh_sigmoid_cross_entropy_grad(n->in1, n->in2, n->out1, n->len1, g_stream));
+}
+// src/gpu/update.cu:56-96
+void k_update(rt::Node* n) { CK(dh_sgd_update(n->out1, n->in1, n->in2, n->len1, g_stream)); }
+void k_moment_update(rt::Node* n) { CK(dh_moment_update(n->out1, n->in1, n->cons1, n->cons2, n->len1, g_stream)); }
+void k_moment_update2(rt::Node* n) { CK(dh_moment_update2(n->out1, n->in1, n->cons1, n->cons2, n->len1, g_stream)); }
+
+// The step counter lives on the host (node->out2) and is advanced at issue time; the corrected
+// rate is formed in float exactly as src/gpu/update.cu:81-93 does.
+float adam_advance(rt::Node* n)
+{
+    dbl_t* t = n->out2;
+    const dbl_t lr = n->cons1, beta1 = n->cons2, beta2 = n->cons3;
+    ++*t;
+    return lr * std::sqrt(1 - std::pow(beta2, *t)) / (1 - std::pow(beta1, *t));
+}
+
+void k_adam_update(rt::Node* n)
+{
+    const float lrt = adam_advance(n);
+    CK(dh_adam_update(n->out1, n->in1, n->in2, lrt, n->cons4, n->len1, g_stream));
+}
+
+// ---- fusion plan -------------------------------------------------------------------------------
+// A step is either one node run through the table or one fused call standing for several nodes.
+struct Step
+{
+    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM } kind = NODE;
+    rt::Node* node = nullptr;    // NODE: the node; CONV_EPILOGUE: the conv node; ACT_BIAS_GRAD: the act-grad node
+    rt::Node* bias = nullptr;    // CONV_EPILOGUE: the mat_rvect_add node (may be null)
+    rt::Node* act = nullptr;     // CONV_EPILOGUE: the activation node (may be null)
+    rt::Node* sum = nullptr;     // ACT_BIAS_GRAD: the mat_sum_cols node
+    rt::Node* m1 = nullptr;      // ADAM: moment_update, moment_update2; node = adam_update
+    rt::Node* m2 = nullptr;
+    const dbl_t* act_ref = nullptr;  // ACT_BIAS_GRAD: tensor the activation gradient reads
+};
+
+int act_code(const rt::Node* n)
+{
+    switch (n->type)
+    {
+    case rt::Node::OP_RELU: return DH_ACT_RELU;
+    case rt::Node::OP_RELU_LEAKY: return DH_ACT_LEAKY;
+    case rt::Node::OP_TANH: return DH_ACT_TANH;
+    case rt::Node::OP_SIGMOID: return DH_ACT_SIGMOID;
+    default: return -1;
+    }
+}
+
+bool is_conv_like(const rt::Node* n)
+{
+    return n->type == rt::Node::OP_CONV2D || n->type == rt::Node::OP_CONV2D_TRANSPOSE ||
+           n->type == rt::Node::OP_CONV2D_TRANSPOSE_INPUT_GRAD || n->type == rt::Node::OP_CONV2D_INPUT_GRAD;
+}
+
+struct Plan
+{
+    std::vector<Step> steps;
+};
+
+// Which instructions of the list read tensor `t`.
+struct Readers
+{
+    std::unordered_map<const dbl_t*, std::vector<rt::Node*>> by_tensor;
+    explicit Readers(const std::vector<rt::Node*>& nodes)
+    {
+        for (rt::Node* n : nodes)
+            for (const dbl_t* t : {n->in1, n->in2, n->in3})
+                if (t)
+                    by_tensor[t].push_back(n);
+    }
+    const std::vector<rt::Node*>& of(const dbl_t* t) const
+    {
+        static const std::vector<rt::Node*> none;
+        auto it = by_tensor.find(t);
+        return it == by_tensor.end() ? none : it->second;
+    }
+};
+
+Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<const dbl_t*>& keep, bool fuse)
+{
+    Plan plan;
+    if (!fuse)
+    {
+        for (rt::Node* n : nodes)
+        {
+            Step s;
+            s.node = n;
+            plan.steps.push_back(s);
+        }
+        return plan;
+    }
+    Readers readers(nodes);
+    std::unordered_set<rt::Node*> absorbed;
+    // activation output that replaces a pre-activation tensor which is no longer materialised
+    std::unordered_map<const dbl_t*, const dbl_t*> z_alias;
+    std::unordered_map<rt::Node*, Step> fused_at;  // fused step keyed by the LAST node it replaces
+
+    auto only_reader = [&](const dbl_t* t, rt::Node* who) {
+        if (keep.count(t))
+            return false;
+        const auto& r = readers.of(t);
+        return r.size() == 1 && r[0] == who;
+    };
+
+    for (rt::Node* n : nodes)
+    {
+        if (absorbed.count(n))
+            continue;
+        if (is_conv_like(n))
+        {
+            // conv -> mat_rvect_add(conv_out, b) [-> activation(z)]
+            rt::Node* bias = nullptr;
+            for (rt::Node* r : readers.of(n->out1))
+                if (r->type == rt::Node::OP_MAT_RVECT_ADD && r->in1 == n->out1)
+                    bias = r;
+            if (!bias || !only_reader(n->out1, bias))
+                continue;
+            Step s;
+            s.kind = Step::CONV_EPILOGUE;
+            s.node = n;
+            s.bias = bias;
+            absorbed.insert(bias);
+            rt::Node* last = bias;
+            // The activation may be folded in when z is read only by it and by gradient nodes that
+            // can take the activation's OUTPUT instead (same sign for relu and for leaky with
+            // alpha > 0), and the caller does not ask for z itself.
+            rt::Node* act = nullptr;
+            bool ok = !keep.count(bias->out1);
+            for (rt::Node* r : readers.of(bias->out1))
+            {
+                const int code = act_code(r);
+                if (code >= 0 && r->in1 == bias->out1 && !act)
+                    act = r;
+                else if ((r->type == rt::Node::OP_RELU_GRAD || r->type == rt::Node::OP_LEAKY_RELU_GRAD) &&
+                         r->in1 == bias->out1 && r->in2 != bias->out1)
+                    ;  // redirected below
+                else
+                    ok = false;
+            }
+            if (ok && act)
+            {
+                const int code = act_code(act);
+                bool sign_safe = true;
+                for (rt::Node* r : readers.of(bias->out1))
+                {
+                    if (r == act)
+                        continue;
+                    if (r->type == rt::Node::OP_RELU_GRAD && code != DH_ACT_RELU)
+                        sign_safe = false;
+                    if (r->type == rt::Node::OP_LEAKY_RELU_GRAD &&
+                        !(code == DH_ACT_LEAKY && act->alpha_leaky > 0.f))
+                        sign_safe = false;
+                }
+                if (sign_safe)
+                {
+                    s.act = act;
+                    absorbed.insert(act);
+                    z_alias[bias->out1] = act->out1;
+                    last = act;
+                }
+            }
+            fused_at[last] = s;
+        }
+    }
+    // activation gradient -> mat_sum_cols, and the three Adam nodes of a variable
+    for (rt::Node* n : nodes)
+    {
+        if (absorbed.count(n))
+            continue;
+        const bool act_grad = n->type == rt::Node::OP_RELU_GRAD || n->type == rt::Node::OP_LEAKY_RELU_GRAD ||
+                              n->type == rt::Node::OP_TANH_GRAD;
+        if (act_grad)
+        {
+            rt::Node* sum = nullptr;
+            for (rt::Node* r : readers.of(n->out1))
+                if (r->type == rt::Node::OP_MAT_SUM_COLS && !absorbed.count(r) && r->len1 * r->len2 == n->len1)
+                    sum = r;
+            if (sum)
+            {
+                Step s;
+                s.kind = Step::ACT_BIAS_GRAD;
+                s.node = n;
+                s.sum = sum;
+                absorbed.insert(n);
+                absorbed.insert(sum);
+                // emitted where the gradient node stood: dz feeds the dk / dx nodes that follow it
+                fused_at[n] = s;
+            }
+        }
+        if (n->type == rt::Node::OP_ADAM_UPDATE)
+        {
+            rt::Node *m1 = nullptr, *m2 = nullptr;
+            for (rt::Node* p : n->preds)
+            {
+                if (p->type == rt::Node::OP_MOMENT_UPDATE && p->out1 == n->in1) m1 = p;
+                if (p->type == rt::Node::OP_MOMENT_UPDATE2 && p->out1 == n->in2) m2 = p;
+            }
+            if (m1 && m2 && m1->in1 == m2->in1 && m1->len1 == n->len1 && m2->len1 == n->len1 &&
+                !absorbed.count(m1) && !absorbed.count(m2) && only_reader(m1->out1, n) && only_reader(m2->out1, n))
+            {
+                Step s;
+                s.kind = Step::ADAM;
+                s.node = n;
+                s.m1 = m1;
+                s.m2 = m2;
+                absorbed.insert(m1);
+                absorbed.insert(m2);
+                absorbed.insert(n);
+                fused_at[n] = s;
+            }
+        }
+    }
+    for (rt::Node* n : nodes)
+    {
+        auto f = fused_at.find(n);
+        if (f != fused_at.end())
+        {
+            Step s = f->second;
+            if (s.kind == Step::ACT_BIAS_GRAD)
+            {
+                auto a = z_alias.find(s.node->in1);
+                s.act_ref = a == z_alias.end() ? s.node->in1 : a->second;
+            }
+            plan.steps.push_back(s);
+            continue;
+        }
+        if (absorbed.count(n))
+            continue;
+        // a conv whose epilogue was fused is emitted at the position of the epilogue's last node
+        bool conv_deferred = false;
+        for (auto& kv : fused_at)
+            if (kv.second.kind == Step::CONV_EPILOGUE && kv.second.node == n)
+                conv_deferred = true;
+        if (conv_deferred)
+            continue;
+        Step s;
+        s.node = n;
+        auto a = (n->type == rt::Node::OP_RELU_GRAD || n->type == rt::Node::OP_LEAKY_RELU_GRAD)
+                     ? z_alias.find(n->in1)
+                     : z_alias.end();
+        s.act_ref = a == z_alias.end() ? nullptr : a->second;
+        plan.steps.push_back(s);
+    }
+    return plan;
+}
+
+void issue(const Step& s)
+{
+    switch (s.kind)
+    {
+    case Step::NODE:
+    {
+        rt::Node* n = s.node;
+        if (s.act_ref)
+        {
+            // gradient of a fused activation: read the activation's output in place of z
+            if (n->type == rt::Node::OP_RELU_GRAD)
+                CK(dh_relu_grad(s.act_ref, n->in2, n->out1, n->len1, g_stream));
+            else
+                CK(dh_leaky_relu_grad(s.act_ref, n->in2, n->out1, n->cons1, n->len1, g_stream));
+            return;
+        }
+        kernel_f f = n->type >= 0 && n->type < 512 ? kernels_list[n->type] : nullptr;
+        if (!f)
+            throw std::runtime_error(std::string("hip backend: operator '") + rt::Node::name_of(n->type) +
+                                     "' is not on the convolution path and has no HIP kernel");
+        f(n);
+        return;
+    }
+    case Step::CONV_EPILOGUE:
+    {
+        rt::Node* c = s.node;
+        const dbl_t* bias = s.bias ? s.bias->in2 : nullptr;
+        const int act = s.act ? act_code(s.act) : DH_ACT_NONE;
+        const float alpha = s.act ? s.act->alpha_leaky : 0.f;
+        dbl_t* out = s.act ? s.act->out1 : s.bias->out1;
+        switch (c->type)
+        {
+        case rt::Node::OP_CONV2D: conv_fwd(geom_conv2d(c), c->in1, c->in2, out, bias, act, alpha); break;
+        case rt::Node::OP_CONV2D_TRANSPOSE: conv_dx(geom_transpose(c), c->in1, c->in2, out, bias, act, alpha); break;
+        case rt::Node::OP_CONV2D_INPUT_GRAD: conv_dx(geom_input_grad(c), c->in1, c->in2, out, bias, act, alpha); break;
+        default: conv_fwd(geom_transpose_input_grad(c), c->in1, c->in2, out, bias, act, alpha); break;
+        }
+        return;
+    }
+    case Step::ACT_BIAS_GRAD:
+    {
+        rt::Node* g = s.node;
+        const int act = g->type == rt::Node::OP_RELU_GRAD ? DH_ACT_RELU
+                        : g->type == rt::Node::OP_LEAKY_RELU_GRAD ? DH_ACT_LEAKY : DH_ACT_TANH;
+        CK(dh_act_bias_grad(s.act_ref, g->in2, g->out1, s.sum->out1, s.sum->len1, s.sum->len2, act, g->cons1,
+                            g_stream));
+        return;
+    }
+    case Step::ADAM:
+    {
+        rt::Node* a = s.node;
+        const float lrt = adam_advance(a);
+        CK(dh_adam_step(a->out1, s.m1->out1, s.m2->out1, s.m1->in1, s.m1->cons1, s.m1->cons2, s.m2->cons1,
+                        s.m2->cons2, lrt, a->cons4, a->len1, g_stream));
+        return;
+    }
+    }
+}
+
+// Plans are cached per instruction list (the lists of a training loop repeat every iteration).
+struct PlanKey
+{
+    std::vector<rt::Node*> nodes;
+    std::vector<const dbl_t*> keep;  // sorted
+    bool fuse;
+    bool operator==(const PlanKey& o) const { return fuse == o.fuse && nodes == o.nodes && keep == o.keep; }
+};
+struct PlanKeyHash
+{
+    std::size_t operator()(const PlanKey& k) const
+    {
+        std::size_t h = k.fuse ? 0x9e3779b97f4a7c15ull : 0;
+        for (rt::Node* n : k.nodes)
+            h = (h ^ reinterpret_cast<std::size_t>(n)) * 0x100000001b3ull;
+        for (const dbl_t* t : k.keep)
+            h = (h ^ reinterpret_cast<std::size_t>(t)) * 0x100000001b3ull;
+        return h;
+    }
+};
+std::unordered_map<PlanKey, Plan, PlanKeyHash> g_plans;
+std::unordered_set<const dbl_t*> g_keep;
+
+}  // namespace
+
+kernel_f kernels_list[512] = {
+    k_mat_mat_mul,                   // 0
+    k_mat_rvect_add,                 // 1
+    k_sigmoid,                       // 2
+    k_mse,                           // 3
+    nullptr,                         // 4  softmax                (not on the convolution path)
+    nullptr,                         // 5  log_softmax            (")
+    nullptr,                         // 6  softmax_cross_entropy  (")
+    k_conv2d,                        // 7
+    k_relu,                          // 8
+    k_relu_leaky,                    // 9
+    k_tanh,                          // 10
+    k_mse_grad,                      // 11
+    k_sigmoid_grad,                  // 12
+    k_mat_mul_add,                   // 13
+    k_tmat_mat_mul,                  // 14
+    k_mat_tmat_mul,                  // 15
+    k_mat_sum_rows,                  // 16
+    k_mat_sum_cols,                  // 17
+    nullptr,                         // 18 softmax_cross_entropy_grad (")
+    k_relu_grad,                     // 19
+    nullptr,                         // 20 conv2d_bias_add: lowered to mat_rvect_add by the operator
+    k_update,                        // 21
+    k_sigmoid_cross_entropy,         // 22
+    k_sigmoid_cross_entropy_grad,    // 23
+    k_conv2d_input_grad,             // 24
+    k_conv2d_kernel_grad,            // 25
+    k_argmax_acc,                    // 26
+    k_moment_update,                 // 27
+    k_moment_update2,                // 28
+    k_adam_update,                   // 29
+    k_leaky_relu_grad,               // 30
+    nullptr,                         // 31 conv2d_bias_add_grad: lowered to mat_sum_cols
+    k_tanh_grad,                     // 32
+    k_conv2d_transpose,              // 33
+    k_conv2d_transpose_input_grad,   // 34
+    k_conv2d_transpose_kernel_grad,  // 35
+    k_add,                           // 36
+};
+
+void set_fusion(bool on)
+{
+    g_fusion = on ? 1 : 0;
+}
+
+bool fusion()
+{
+    if (g_fusion < 0)
+    {
+        const char* env = std::getenv("DCGAN_HIP_FUSE");
+        g_fusion = env && !std::strcmp(env, "1") ? 1 : 0;
+    }
+    return g_fusion == 1;
+}
+
+namespace { bool g_sync_each_run = true; }
+void set_sync_each_run(bool on) { g_sync_each_run = on; }
+bool sync_each_run() { return g_sync_each_run; }
+
+void* stream() { return g_stream; }
+
+void synchronize() { CK(dh_stream_sync(g_stream)); }
+
+void set_protected_tensors(const std::vector<const dbl_t*>& tensors)
+{
+    g_keep.clear();
+    g_keep.insert(tensors.begin(), tensors.end());
+}
+
+void run_async(rt::NodesList& tasks)
+{
+    PlanKey key{tasks.nodes(), std::vector<const dbl_t*>(g_keep.begin(), g_keep.end()), fusion()};
+    std::sort(key.keep.begin(), key.keep.end());
+    auto it = g_plans.find(key);
+    if (it == g_plans.end())
+        it = g_plans.emplace(key, make_plan(tasks.nodes(), g_keep, key.fuse)).first;
+    for (const Step& s : it->second.steps)
+        issue(s);
+}
+
+void run(rt::NodesList& tasks)
+{
+    run_async(tasks);
+    synchronize();
+}
+
+void forget_plans()
+{
+    g_plans.clear();
+}
+
+}  // namespace hip
+
+namespace rt
+{
+namespace
+{
+runner_f g_cpu[2] = {nullptr, nullptr};
+}
+
+void register_cpu_backend(ProgramMode mode, runner_f runner)
+{
+    if (mode == ProgramMode::MONOTHREAD) g_cpu[0] = runner;
+    if (mode == ProgramMode::MULTITHREAD) g_cpu[1] = runner;
+}
+
+void execute(NodesList& tasks)
+{
+    const ProgramMode mode = program_mode();
+    if (mode == ProgramMode::GPU)
+    {
+        if (hip::sync_each_run())
+            hip::run(tasks);
+        else
+            hip::run_async(tasks);
+        return;
+    }
+    runner_f r = g_cpu[mode == ProgramMode::MONOTHREAD ? 0 : 1];
+    if (!r)
+        throw std::runtime_error(
+            "RT_MODE selects a CPU mode, but this library only holds the HIP backend (RT_MODE=GPU); "
+            "the CPU runners are the reference's src/cpu tree -- register one with rt::register_cpu_backend");
+    r(tasks);
+}
+}  // namespace rt

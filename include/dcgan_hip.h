@@ -68,6 +68,14 @@ int dh_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop`
 int dh_workspace_reserve(size_t bytes);
 size_t dh_workspace_bytes(void);
 
+/* Per-kernel timing of the convolution kernels (no counterpart in the reference, whose only timer
+ * is the per-run wall clock of src/ops/graph.cu:150-169).  While enabled, every implicit-GEMM
+ * launch is bracketed by HIP events on its stream.  dh_profile_read() waits for them and writes one
+ * line per kernel instantiation: "name<TAB>launches<TAB>total ms<TAB>total algorithmic FLOPs". */
+int dh_profile_enable(int on);
+int dh_profile_reset(void);
+int dh_profile_read(char* buf, size_t buf_len);
+
 /* ---- convolutions: fp32 implicit GEMM on MFMA, no im2col buffer ------------------------------ */
 
 /* conv2d forward, optionally with the bias add and activation that follow it fused in.
@@ -173,10 +181,12 @@ int dh_moment_update2(float* v, const float* g, float a, float b, size_t n, void
 /* p -= lrt * m / (sqrt(v) + eps); lrt = lr*sqrt(1-beta2^t)/(1-beta1^t) is formed by the caller on
  * the host in float, as the reference does (src/gpu/update.cu:81-96). */
 int dh_adam_update(float* p, const float* m, const float* v, float lrt, float eps, size_t n, void* stream);
-/* The three kernels above in one pass (28 B/param instead of 40): m, v and p are updated in place
- * with the same arithmetic, in the same order, as the three separate calls. */
-int dh_adam_step(float* p, float* m, float* v, const float* g, float beta1, float beta2,
-                 float lrt, float eps, size_t n, void* stream);
+/* The three kernels above in one pass (28 B/param instead of 40):
+ *   m = m_decay*m + m_gain*g;  v = v_decay*v + v_gain*g*g;  p -= lrt * m / (sqrt(v) + eps)
+ * with the same arithmetic, in the same order, as the three separate calls
+ * (the reference passes beta and 1 - beta, src/api/adam-optimizer.cu:48-49). */
+int dh_adam_step(float* p, float* m, float* v, const float* g, float m_decay, float m_gain,
+                 float v_decay, float v_gain, float lrt, float eps, size_t n, void* stream);
 /* var += *coeff * dv with coeff a DEVICE scalar.  Replaces gpu::vect_update (src/gpu/update.cu:14-21). */
 int dh_sgd_update(float* var, const float* dv, const float* coeff_device, size_t n, void* stream);
 

@@ -1,0 +1,81 @@
+"""Whole-network parity, layer by layer, in the manner of the reference's test_dcgan_generator /
+test_dcgan_discriminator (which export every layer, the loss and all dW/db): the DCGAN evaluated
+through the operator graph on the HIP backend against the same graph on the CPU oracle backend,
+on identical seeded weights and inputs -- unfused and with the fused launches."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import dcgan_reference as dr
+from common import RTOL, ATOL
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BATCH, SEED = 2, 7
+
+
+@pytest.fixture(scope="module")
+def cpu_dump(tmp_path_factory):
+    path = str(tmp_path_factory.mktemp("dcgan") / "cpu.npz")
+    env = dict(os.environ, RT_MODE="CPU", OMP_NUM_THREADS="16")
+    subprocess.run([sys.executable, os.path.join(ROOT, "tests", "dcgan_reference.py"), str(BATCH), str(SEED), path],
+                   check=True, env=env, timeout=600)
+    return dict(np.load(path))
+
+
+def gpu_dump(fusion):
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    model = pkg.hostabi.DcganModel(BATCH, SEED, "GPU")
+    try:
+        model.set_fusion(fusion)
+        w, z, x = dr.synthetic(BATCH, SEED, pkg.hostabi.var_shapes())
+        for name, val in w.items():
+            model.set_var(name, val)
+        model.set_inputs(z, x)
+        return dr.collect(model), model.last_schedule_size()
+    finally:
+        model.set_fusion(False)
+        model.close()
+
+
+@pytest.mark.parametrize("fusion", [False, True])
+def test_dcgan_layers_losses_gradients_and_one_adam_iteration(cpu_dump, fusion):
+    print("fusion", fusion, flush=True)
+    got, _ = gpu_dump(fusion)
+    assert set(got) == set(cpu_dump)
+    for key in sorted(cpu_dump):
+        exp = cpu_dump[key].reshape(-1)
+        g = got[key].reshape(-1)
+        if key.startswith("after_"):
+            # parameters after one Adam step: the step is lr*m/(sqrt(v)+eps) ~ lr*sign(g); where a
+            # gradient is ~0 its sign is noise, so compare with the step size as absolute tolerance
+            np.testing.assert_allclose(g, exp, rtol=RTOL, atol=4.1e-4, err_msg=key)
+            assert np.mean(np.abs(g - exp) > 1e-5) < 0.02, key
+        else:
+            scale = max(1.0, float(np.abs(exp).max()))
+            np.testing.assert_allclose(g, exp, rtol=RTOL, atol=ATOL * scale, err_msg=key)
+
+
+def test_generate_and_argmax_bit_exact(cpu_dump):
+    """The generated images agree to tolerance and their per-pixel argmax over channels is identical."""
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    model = pkg.hostabi.DcganModel(BATCH, SEED, "GPU")
+    try:
+        w, z, x = dr.synthetic(BATCH, SEED, pkg.hostabi.var_shapes())
+        for name, val in w.items():
+            model.set_var(name, val)
+        model.set_inputs(z, x)
+        img = model.generate()
+    finally:
+        model.close()
+    exp = cpu_dump["g_out"].reshape(img.shape)
+    np.testing.assert_allclose(img, exp, rtol=RTOL, atol=ATOL)
+    margin = np.sort(exp, axis=-1)
+    clear = (margin[..., -1] - margin[..., -2]) > 1e-5   # exclude numerical ties
+    assert np.array_equal(img.argmax(-1)[clear], exp.argmax(-1)[clear])
+    assert clear.mean() > 0.95
