@@ -1,7 +1,7 @@
 // Dense-layer products of the DCGAN (z -> 4*4*512 and 8192 -> 1, and their gradients): well under
 // 1 % of an iteration's FLOPs, so a compact LDS-tiled FMA kernel with strided operand views covers
 // A*B, tr(A)*B and A*tr(B); tall-skinny products with few outputs and a long contraction (8192 -> 1)
-// use one wavefront per output instead.
+// use one workgroup per output instead.
 //
 // Reference counterparts: src/gpu/matmul.cu:12-86 (one thread per output, no tiling).
 #include "dh_common.h"
@@ -65,22 +65,27 @@ __global__ __launch_bounds__(256) void gemm_tiled(const float* __restrict__ a, c
         }
 }
 
-// one wavefront per output element, lanes stride over k, fixed shuffle tree
-__global__ __launch_bounds__(256) void gemm_wave_per_output(const float* __restrict__ a, const float* __restrict__ b,
-                                                            const float* __restrict__ bias, float* __restrict__ out,
-                                                            int M, int K, int P, size_t sai, size_t sak, size_t sbk,
-                                                            size_t sbj)
+// one workgroup per output element: 256 lanes stride over k, then a fixed LDS tree
+__global__ __launch_bounds__(256) void gemm_block_per_output(const float* __restrict__ a, const float* __restrict__ b,
+                                                             const float* __restrict__ bias, float* __restrict__ out,
+                                                             int M, int K, int P, size_t sai, size_t sak, size_t sbk,
+                                                             size_t sbj)
 {
-    const size_t o = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
-    if (o >= (size_t)M * P) return;
+    __shared__ float lds[256];
+    const size_t o = blockIdx.x;
     const int i = (int)(o / P), j = (int)(o % P);
     float s = 0.f;
-    for (int k = lane; k < K; k += 64)
+    for (int k = threadIdx.x; k < K; k += 256)
         s += a[(size_t)i * sai + (size_t)k * sak] * b[(size_t)k * sbk + (size_t)j * sbj];
-    for (int off = 32; off > 0; off >>= 1)
-        s += __shfl_down(s, off, 64);
-    if (lane == 0) out[o] = s + (bias ? bias[j] : 0.f);
+    lds[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1)
+    {
+        if ((int)threadIdx.x < w) lds[threadIdx.x] += lds[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[o] = lds[0] + (bias ? bias[j] : 0.f);
+    (void)M;
 }
 
 int run_gemm(const char* who, const float* a, const float* b, const float* bias, float* out, size_t m, size_t n,
@@ -92,7 +97,7 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     if (m > 0x7fffffff || n > 0x7fffffff || p > 0x7fffffff) return fail(DH_EINVAL, "%s: extent too large", who);
     hipStream_t st = as_stream(stream);
     if (m * p <= 4096 && n >= 512)
-        hipLaunchKernelGGL(gemm_wave_per_output, dim3((unsigned)((m * p + 3) / 4)), dim3(256), 0, st, a, b, bias, out,
+        hipLaunchKernelGGL(gemm_block_per_output, dim3((unsigned)(m * p)), dim3(256), 0, st, a, b, bias, out,
                            (int)m, (int)n, (int)p, sai, sak, sbk, sbj);
     else
         hipLaunchKernelGGL(gemm_tiled, dim3((unsigned)((p + TS - 1) / TS), (unsigned)((m + TS - 1) / TS)), dim3(256), 0,

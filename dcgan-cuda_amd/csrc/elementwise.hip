@@ -246,15 +246,20 @@ __global__ __launch_bounds__(TPB) void colsum_stage1(const float* __restrict__ a
     }
 }
 
+// One wavefront per column: lane l adds the per-range sums l, l+64, ... in that order, then the 64
+// lane sums are combined by a fixed shuffle tree.
 __global__ __launch_bounds__(TPB) void colsum_stage2(const float* __restrict__ partial, float* __restrict__ out,
                                                      uint32_t cols, uint32_t chunks)
 {
-    const uint32_t c = blockIdx.x * TPB + threadIdx.x;
+    const uint32_t c = blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
+    const uint32_t lane = threadIdx.x & 63;
     if (c >= cols) return;
     float s = 0.f;
-    for (uint32_t q = 0; q < chunks; ++q)
+    for (uint32_t q = lane; q < chunks; q += 64)
         s += partial[(size_t)q * cols + c];
-    out[c] = s;
+    for (int off = 32; off > 0; off >>= 1)
+        s += __shfl_down(s, off, 64);
+    if (lane == 0) out[c] = s;
 }
 
 int run_colsum(const char* who, const float* a, const float* act_ref, float* dz, float* db, size_t rows,
@@ -302,8 +307,8 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     DH_LAUNCH_CHECK(who);
     if (db)
     {
-        hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + TPB - 1) / TPB)), dim3(TPB), 0, st, partial,
-                           db, (uint32_t)cols, (uint32_t)chunks);
+        hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + TPB / 64 - 1) / (TPB / 64))), dim3(TPB), 0, st,
+                           partial, db, (uint32_t)cols, (uint32_t)chunks);
         DH_LAUNCH_CHECK(who);
     }
     return 0;
