@@ -409,6 +409,331 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm(const ConvParams p)
         }
 }
 
+// ---- fast path -------------------------------------------------------------------------------------
+// Same tiling and arithmetic as conv_igemm, for the common case where every 4-chunk can be loaded as
+// one 16-byte access (channel counts divisible by 4, 16-byte aligned tensors of less than 2^31
+// bytes).  What changes is how operands are fetched:
+//   * the part of an address that depends on the tile row (image, output pixel) is decoded ONCE per
+//     thread before the k loop; per k-slab only the filter tap is decoded, once per thread;
+//   * loads go through buffer descriptors: an element that falls into the padding, past the end of
+//     the contraction or outside the tile gets an out-of-range offset and the hardware returns 0,
+//     so the loop body has no branches and the compiler can interleave address arithmetic, LDS
+//     traffic and MFMA in one basic block.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int32_t OOB = (int32_t)0x80000000u;  // any offset >= num_records reads as zero
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const float* ptr, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ptr), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, int32_t byte_off)
+{
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0));
+}
+
+template <int MODE, int BM, int BN, int WGM, int WGN>
+__global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, uint32_t a_bytes, uint32_t b_bytes)
+{
+    static_assert(WGM * WGN == 4, "four wavefronts per workgroup");
+    constexpr bool A_KC = MODE != MODE_DK;
+    constexpr bool B_KC = MODE == MODE_DX;
+    constexpr int WM = BM / WGM, WN = BN / WGN;
+    constexpr int TM = WM / 32, TN = WN / 32;
+    using TA = Tile<A_KC, BM>;
+    using TB = Tile<B_KC, BN>;
+    constexpr int NA = TA::PER_THREAD, NB = TB::PER_THREAD;
+
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TA::SIZE];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][TB::SIZE];
+
+    const Phase& ph = p.phase[blockIdx.z];
+    const int tiles_n = (p.ncols + BN - 1) / BN;
+    const int tile_m = blockIdx.x / tiles_n;
+    const int tile_n = blockIdx.x - tile_m * tiles_n;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    if (m0 >= ph.M)
+        return;
+
+    const int nslabs = (ph.K + BK - 1) / BK;
+    const int per_split = (nslabs + p.splitk - 1) / p.splitk;
+    const int s_begin = blockIdx.y * per_split;
+    const int s_end = min(nslabs, s_begin + per_split);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
+
+    const __amdgpu_buffer_rsrc_t ra_src = make_rsrc(p.a_src, a_bytes);
+    const __amdgpu_buffer_rsrc_t rb_src = make_rsrc(p.b_src, b_bytes);
+
+    // ---- per-thread state that does not depend on k -------------------------------------------------
+    // K-contiguous operand tiles: chunk q of this thread is row (tid + q*256) / 4, k offset (tid % 4) * 4.
+    // Other tiles: chunk q is k row tid / (R/4) + q * 256/(R/4), row offset (tid % (R/4)) * 4.
+    const int kloc = (tid % (BK / 4)) * 4;
+    int a_base[NA], a_h[NA], a_w[NA];   // FWD/DX: byte offset of the row's origin, its (h, w) origin
+    int a_krow[NA];                      // DK: k row of the chunk inside the slab
+    int a_moff = 0, a_dh = 0, a_dw = 0;  // DK: per-thread filter tap (byte offset, h and w shifts)
+    bool a_mvalid = true;
+#pragma unroll
+    for (int q = 0; q < NA; ++q)
+    {
+        const int idx = tid + q * NTHREADS;
+        a_base[q] = 0; a_h[q] = 0; a_w[q] = 0; a_krow[q] = 0;
+        if (A_KC)
+        {
+            const int m = m0 + idx / (BK / 4);
+            const bool live = m < ph.M && idx < TA::CHUNKS;
+            uint32_t b = 0, rem = 0, r1 = 0, r2 = 0;
+            if (MODE == MODE_FWD)
+            {
+                p.fd_HoWo.divmod(live ? m : 0, b, rem);
+                p.fd_Wo.divmod(rem, r1, r2);
+                a_h[q] = (int)r1 * p.sh - p.pt;
+                a_w[q] = (int)r2 * p.sw - p.pl;
+                a_base[q] = (((int)b * p.H + a_h[q]) * p.W + a_w[q]) * p.C * 4;
+            }
+            else
+            {
+                ph.fd_HpWp.divmod(live ? m : 0, b, rem);
+                ph.fd_Wp.divmod(rem, r1, r2);
+                a_h[q] = (int)r1 + ph.q0h;
+                a_w[q] = (int)r2 + ph.q0w;
+                a_base[q] = (((int)b * p.Ho + a_h[q]) * p.Wo + a_w[q]) * p.O * 4;
+            }
+            if (!live)
+                a_h[q] = -(1 << 28);  // fails every bounds check
+        }
+        else
+            a_krow[q] = idx / (BM / 4);
+    }
+    if (!A_KC)
+    {
+        const int mc = m0 + (tid % (BM / 4)) * 4;
+        a_mvalid = mc < ph.M;
+        uint32_t tap, c, di, dj;
+        p.fd_C.divmod(a_mvalid ? mc : 0, tap, c);
+        p.fd_kw.divmod(tap, di, dj);
+        a_dh = (int)di - p.pt;
+        a_dw = (int)dj - p.pl;
+        a_moff = ((a_dh * p.W + a_dw) * p.C + (int)c) * 4;
+    }
+
+    int b_off[NB];  // FWD/DK: running byte offset; DX: byte offset of the row (output channel)
+#pragma unroll
+    for (int q = 0; q < NB; ++q)
+    {
+        const int idx = tid + q * NTHREADS;
+        if (B_KC)
+        {
+            const int n = n0 + idx / (BK / 4);
+            b_off[q] = (n < p.ncols && idx < TB::CHUNKS) ? n * p.O * 4 : OOB;
+        }
+        else
+        {
+            const int n = n0 + (tid % (BN / 4)) * 4;
+            const int krow = idx / (BN / 4);
+            b_off[q] = (n < p.ncols && idx < TB::CHUNKS) ? ((s_begin * BK + krow) * p.ncols + n) * 4 : OOB;
+        }
+    }
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[a][b][r] = 0.f;
+
+    f32x4 ra[NA], rb[NB];
+
+    auto load_global = [&](int slab) {
+        const int k0 = slab * BK;
+        // decode of the k coordinate shared by all chunks of this thread
+        int ka_off = 0, ka_d0 = 0, ka_d1 = 0, kb_off = 0;
+        bool kvalid = true;
+        if (MODE == MODE_FWD)
+        {
+            const int kk = k0 + kloc;
+            kvalid = kk < ph.K;
+            uint32_t tap, c, di, dj;
+            p.fd_C.divmod(kvalid ? kk : 0, tap, c);
+            p.fd_kw.divmod(tap, di, dj);
+            ka_d0 = (int)di; ka_d1 = (int)dj;
+            ka_off = (((int)di * p.W + (int)dj) * p.C + (int)c) * 4;
+        }
+        else if (MODE == MODE_DX)
+        {
+            const int kk = k0 + kloc;
+            kvalid = kk < ph.K;
+            uint32_t tap, o, th, tw;
+            p.fd_O.divmod(kvalid ? kk : 0, tap, o);
+            ph.fd_ntw.divmod(tap, th, tw);
+            ka_d0 = -(int)th; ka_d1 = -(int)tw;
+            ka_off = ((int)o - ((int)th * p.Wo + (int)tw) * p.O) * 4;
+            kb_off = ((((ph.rh + p.sh * (int)th) * p.kw + ph.rw + p.sw * (int)tw) * p.C) * p.O + (int)o) * 4;
+        }
+#pragma unroll
+        for (int q = 0; q < NA; ++q)
+        {
+            int off;
+            if (A_KC)
+            {
+                const int lim_h = MODE == MODE_FWD ? p.H : p.Ho, lim_w = MODE == MODE_FWD ? p.W : p.Wo;
+                const bool ok = kvalid && (unsigned)(a_h[q] + ka_d0) < (unsigned)lim_h &&
+                                (unsigned)(a_w[q] + ka_d1) < (unsigned)lim_w;
+                off = ok ? a_base[q] + ka_off : OOB;
+            }
+            else
+            {
+                const int kk = k0 + a_krow[q];
+                const bool kin = kk < ph.K;
+                uint32_t b, rem, i, j;
+                p.fd_HoWo.divmod(kin ? kk : 0, b, rem);
+                p.fd_Wo.divmod(rem, i, j);
+                const int h = (int)i * p.sh, w = (int)j * p.sw;
+                const bool ok = kin && a_mvalid && (unsigned)(h + a_dh) < (unsigned)p.H &&
+                                (unsigned)(w + a_dw) < (unsigned)p.W && (tid + q * NTHREADS) < TA::CHUNKS;
+                off = ok ? (((int)b * p.H + h) * p.W + w) * p.C * 4 + a_moff : OOB;
+            }
+#ifdef EXP_NO_GLOBAL
+            off = OOB;
+#endif
+            ra[q] = buf_load4(ra_src, off);
+        }
+#pragma unroll
+        for (int q = 0; q < NB; ++q)
+        {
+            int off;
+            if (B_KC)
+                off = (kvalid && b_off[q] != OOB) ? b_off[q] + kb_off : OOB;
+            else
+            {
+                off = b_off[q];  // rows past the end of the contraction lie past the end of the buffer
+                if (b_off[q] != OOB)
+                    b_off[q] += BK * p.ncols * 4;
+            }
+#ifdef EXP_NO_GLOBAL
+            off = OOB;
+#endif
+            rb[q] = buf_load4(rb_src, off);
+        }
+    };
+    auto store_lds = [&](int stage) {
+#pragma unroll
+        for (int q = 0; q < NA; ++q)
+        {
+            const int idx = tid + q * NTHREADS;
+            if (TA::CHUNKS % NTHREADS == 0 || idx < TA::CHUNKS)
+            {
+                int row, k;
+                TA::chunk(idx, row, k);
+                TA::store(lds_a[stage], row, k, make_float4(ra[q].x, ra[q].y, ra[q].z, ra[q].w));
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NB; ++q)
+        {
+            const int idx = tid + q * NTHREADS;
+            if (TB::CHUNKS % NTHREADS == 0 || idx < TB::CHUNKS)
+            {
+                int row, k;
+                TB::chunk(idx, row, k);
+                TB::store(lds_b[stage], row, k, make_float4(rb[q].x, rb[q].y, rb[q].z, rb[q].w));
+            }
+        }
+    };
+
+    if (s_begin < s_end)
+    {
+        load_global(s_begin);
+        store_lds(0);
+        __syncthreads();
+        for (int s = s_begin; s < s_end; ++s)
+        {
+            const int stage = (s - s_begin) & 1;
+            if (s + 1 < s_end)
+                load_global(s + 1);
+            float4 fa[2][TM], fb[2][TN];
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+                fa[0][a] = TA::frag(lds_a[stage], wm0 + a * 32 + l32, 0, half);
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+                fb[0][b] = TB::frag(lds_b[stage], wn0 + b * 32 + l32, 0, half);
+#pragma unroll
+            for (int kg = 0; kg < BK / 8; ++kg)
+            {
+                const int cur = kg & 1;
+                if (kg + 1 < BK / 8)
+                {
+#pragma unroll
+                    for (int a = 0; a < TM; ++a)
+                        fa[cur ^ 1][a] = TA::frag(lds_a[stage], wm0 + a * 32 + l32, kg + 1, half);
+#pragma unroll
+                    for (int b = 0; b < TN; ++b)
+                        fb[cur ^ 1][b] = TB::frag(lds_b[stage], wn0 + b * 32 + l32, kg + 1, half);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int a = 0; a < TM; ++a)
+#pragma unroll
+                        for (int b = 0; b < TN; ++b)
+                            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                reinterpret_cast<const float*>(&fa[cur][a])[j],
+                                reinterpret_cast<const float*>(&fb[cur][b])[j], acc[a][b], 0, 0, 0);
+            }
+#ifdef EXP_NO_LDS_STORE
+            if (s + 1 < s_end && ra[0].x == 12345.f)
+#else
+            if (s + 1 < s_end)
+#endif
+                store_lds(stage ^ 1);
+            __syncthreads();
+        }
+    }
+
+    const bool direct = p.splitk == 1;
+    float* dst = direct ? p.out : p.part + (size_t)blockIdx.y * p.out_elems;
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+        {
+            const int m = m0 + wm0 + a * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+            if (m >= ph.M)
+                continue;
+            size_t row_off;
+            if (MODE == MODE_DX)
+            {
+                uint32_t b, rem, hh, ww;
+                ph.fd_HpWp.divmod(m, b, rem);
+                ph.fd_Wp.divmod(rem, hh, ww);
+                row_off = (((size_t)b * p.H + hh * p.sh + ph.ph) * p.W + ww * p.sw + ph.pw) * p.C;
+            }
+            else
+                row_off = (size_t)m * p.ncols;
+#pragma unroll
+            for (int b = 0; b < TN; ++b)
+            {
+                const int n = n0 + wn0 + b * 32 + l32;
+                if (n >= p.ncols)
+                    continue;
+                float v = acc[a][b][r];
+                if (direct)
+                {
+                    if (p.bias)
+                        v += p.bias[n];
+                    v = apply_act(v, p.act, p.alpha);
+                }
+                dst[row_off + n] = v;
+            }
+        }
+}
+
 // out[i] = act(bias[i % cols] + sum_s part[s][i]) -- the partial sums are added in split order, so
 // the result does not depend on which workgroup finished first.
 template <bool VEC>
@@ -501,22 +826,34 @@ hipEvent_t prof_event()
     return e;
 }
 
+// Bytes of the two operand tensors, for the buffer descriptors of the fast path (0 = too large).
+struct OperandBytes { size_t a, b; };
+OperandBytes g_operand_bytes = {0, 0};
+bool g_force_generic = false;  // tests: exercise the general kernel on shapes the fast one would take
+
 template <int MODE, int BM, int BN, int WGM, int WGN>
 int launch_cfg(const ConvParams& p, dim3 grid, bool veca, bool vecb, hipStream_t st)
 {
+    const bool fast = veca && vecb && !g_force_generic && g_operand_bytes.a > 0 && g_operand_bytes.b > 0 &&
+                      g_operand_bytes.a < (size_t(1) << 31) && g_operand_bytes.b < (size_t(1) << 31);
     ProfRecord rec{};
     if (g_prof_on)
     {
         char name[96];
         snprintf(name, sizeof(name), "conv_igemm<%s,%dx%d,%s%s>", MODE == MODE_FWD ? "fwd" : MODE == MODE_DX ? "dx" : "dk",
                  BM, BN, veca ? "v" : "s", vecb ? "v" : "s");
+        if (fast)
+            snprintf(name, sizeof(name), "conv_igemm_fast<%s,%dx%d>", MODE == MODE_FWD ? "fwd" : MODE == MODE_DX ? "dx" : "dk", BM, BN);
         rec.tag = prof_tag(name);
         rec.flops = g_prof_flops;
         rec.e0 = prof_event();
         rec.e1 = prof_event();
         (void)hipEventRecord(rec.e0, st);
     }
-    if (veca && vecb)
+    if (fast)
+        hipLaunchKernelGGL((conv_igemm_fast<MODE, BM, BN, WGM, WGN>), grid, dim3(NTHREADS), 0, st, p,
+                           (uint32_t)g_operand_bytes.a, (uint32_t)g_operand_bytes.b);
+    else if (veca && vecb)
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, true, true>), grid, dim3(NTHREADS), 0, st, p);
     else if (veca)
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, true, false>), grid, dim3(NTHREADS), 0, st, p);
@@ -648,6 +985,7 @@ int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W,
     const bool veca = C % 4 == 0 && aligned16(x);
     const bool vecb = O % 4 == 0 && aligned16(k);
     g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C;
+    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)kh * kw * C * O * 4};
     DH_TRY(run_igemm<MODE_FWD>(p, 1, p.phase[0].M, veca, vecb, as_stream(stream), cfg));
     return finish_splitk(p, as_stream(stream));
 }
@@ -707,6 +1045,7 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
     const bool vecb = O % 4 == 0 && aligned16(k);
     // one launch covers up to MAX_PHASES phases; the operator's FLOPs are split evenly over launches
     g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C / ((n_live + MAX_PHASES - 1) / MAX_PHASES > 0 ? (n_live + MAX_PHASES - 1) / MAX_PHASES : 1);
+    g_operand_bytes = {(size_t)N * Ho * Wo * O * 4, (size_t)kh * kw * C * O * 4};
     for (int z0 = 0; z0 < n_live; z0 += MAX_PHASES)
     {
         const int nz = n_live - z0 < MAX_PHASES ? n_live - z0 : MAX_PHASES;
@@ -746,10 +1085,17 @@ int dh_conv2d_dk(const float* x, const float* dy, float* dk, int N, int H, int W
     const bool veca = C % 4 == 0 && aligned16(x);
     const bool vecb = O % 4 == 0 && aligned16(dy);
     g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C;
+    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)N * Ho * Wo * O * 4};
     DH_TRY(run_igemm<MODE_DK>(p, 1, p.phase[0].M, veca, vecb, as_stream(stream), cfg));
     return finish_splitk(p, as_stream(stream));
 }
 
+
+int dh_debug_force_generic_conv(int on)
+{
+    g_force_generic = on != 0;
+    return 0;
+}
 
 int dh_profile_enable(int on)
 {

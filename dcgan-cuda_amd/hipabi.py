@@ -12,7 +12,8 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libdcgan_hip.so")
+# DCGAN_HIP_LIB overrides the library file (A/B runs of an experimental build)
+LIB_PATH = os.environ.get("DCGAN_HIP_LIB") or os.path.join(HERE, "lib", "libdcgan_hip.so")
 
 ACT_NONE, ACT_RELU, ACT_LEAKY, ACT_TANH, ACT_SIGMOID = range(5)
 
@@ -37,6 +38,7 @@ _SIGS = {
     "dh_event_record": [_vp, _vp],
     "dh_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "dh_workspace_reserve": [_sz],
+    "dh_debug_force_generic_conv": [_i],
     "dh_profile_enable": [_i],
     "dh_profile_reset": [],
     "dh_profile_read": [C.c_char_p, _sz],

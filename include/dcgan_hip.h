@@ -76,6 +76,10 @@ int dh_profile_enable(int on);
 int dh_profile_reset(void);
 int dh_profile_read(char* buf, size_t buf_len);
 
+/* Test hook: on != 0 routes every convolution through the general kernel (element-wise bounds
+ * checks, any channel count or alignment) even where the 16-byte buffer-load kernel applies. */
+int dh_debug_force_generic_conv(int on);
+
 /* ---- convolutions: fp32 implicit GEMM on MFMA, no im2col buffer ------------------------------ */
 
 /* conv2d forward, optionally with the bias add and activation that follow it fused in.

@@ -86,6 +86,24 @@ def test_fused_epilogues(be, orc, act, shape):
           f(orc.bias_add(orc.conv2d_input_grad(dy, k, s, (H, W)), bc)))
 
 
+@pytest.mark.parametrize("shape", [(5, 12, 12, 36, 5, 5, 72, 2), (2, 32, 32, 64, 5, 5, 128, 2), (4, 8, 8, 256, 5, 5, 512, 2)])
+def test_general_kernel_on_vector_shapes(be, orc, shape):
+    """Shapes that normally take the 16-byte buffer-load kernel, forced through the general kernel
+    (element-wise bounds checks), so that both code paths stay covered."""
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(11, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    orc.set_threads(8)
+    be.lib.dh_debug_force_generic_conv(1)
+    try:
+        close(be.conv2d(x, k, (s, s)), orc.conv2d(x, k, (s, s)), what="fwd")
+        close(be.conv2d_input_grad(dy, k, s, (H, W)), orc.conv2d_input_grad(dy, k, s, (H, W)), what="dx")
+        exp = orc.conv2d_kernel_grad(dy, x, s, pads)
+        close(be.conv2d_kernel_grad(dy, x, s, pads), exp, scale=max(1.0, float(np.abs(exp).max())), what="dk")
+    finally:
+        be.lib.dh_debug_force_generic_conv(0)
+
+
 def test_dk_is_reproducible(be):
     """Split-K partial sums are reduced in a fixed order: two runs give identical bits."""
     x, k, dy = rand_conv_inputs(3, 8, 16, 16, 128, 5, 5, 256, 2)
