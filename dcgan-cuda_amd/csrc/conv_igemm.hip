@@ -41,7 +41,7 @@ struct Phase
     int Hp, Wp;          // DX: output rows/cols in this phase
     int rh, rw;          // DX: first filter tap of the phase
     int q0h, q0w;        // DX: i = hh + q0h - th
-    int ntw;             // DX: taps along w
+    int nth, ntw;        // DX: taps along h and w
     FastDiv fd_HpWp, fd_Wp, fd_ntw;
 };
 
@@ -488,7 +488,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
             uint32_t b = 0, rem = 0, r1 = 0, r2 = 0;
             if (MODE == MODE_FWD)
             {
-                p.fd_HoWo.divmod(live ? m : 0, b, rem);
+                p.fd_HoWo.divmod(m, b, rem);
                 p.fd_Wo.divmod(rem, r1, r2);
                 a_h[q] = (int)r1 * p.sh - p.pt;
                 a_w[q] = (int)r2 * p.sw - p.pl;
@@ -496,7 +496,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
             }
             else
             {
-                ph.fd_HpWp.divmod(live ? m : 0, b, rem);
+                ph.fd_HpWp.divmod(m, b, rem);
                 ph.fd_Wp.divmod(rem, r1, r2);
                 a_h[q] = (int)r1 + ph.q0h;
                 a_w[q] = (int)r2 + ph.q0w;
@@ -513,7 +513,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
         const int mc = m0 + (tid % (BM / 4)) * 4;
         a_mvalid = mc < ph.M;
         uint32_t tap, c, di, dj;
-        p.fd_C.divmod(a_mvalid ? mc : 0, tap, c);
+        p.fd_C.divmod(mc, tap, c);
         p.fd_kw.divmod(tap, di, dj);
         a_dh = (int)di - p.pt;
         a_dw = (int)dj - p.pl;
@@ -547,9 +547,14 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
             for (int r = 0; r < 16; ++r)
                 acc[a][b][r] = 0.f;
 
-    f32x4 ra[NA], rb[NB];
+    // Two register sets: a slab's loads are issued one slab time before its data is needed in LDS.
+    f32x4 ra0[NA], rb0[NB], ra1[NA], rb1[NB];
 
-    auto load_global = [&](int slab) {
+    // Issues the loads of one k-slab into a register set.  Nothing in here may turn into a branch
+    // (the compiler counts outstanding loads exactly only in straight-line code): validity tests use
+    // the decoded tap rather than k itself and are combined with bitwise AND, divisions run
+    // unconditionally (dh::FastDiv is total on [0, 2^31)), slabs past s_end get out-of-range offsets.
+    auto load_global = [&](f32x4* ra, f32x4* rb, int slab) {
         const int k0 = slab * BK;
         // decode of the k coordinate shared by all chunks of this thread
         int ka_off = 0, ka_d0 = 0, ka_d1 = 0, kb_off = 0;
@@ -557,20 +562,20 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
         if (MODE == MODE_FWD)
         {
             const int kk = k0 + kloc;
-            kvalid = kk < ph.K;
             uint32_t tap, c, di, dj;
-            p.fd_C.divmod(kvalid ? kk : 0, tap, c);
+            p.fd_C.divmod(kk, tap, c);
             p.fd_kw.divmod(tap, di, dj);
+            kvalid = (int)di < p.kh;
             ka_d0 = (int)di; ka_d1 = (int)dj;
             ka_off = (((int)di * p.W + (int)dj) * p.C + (int)c) * 4;
         }
         else if (MODE == MODE_DX)
         {
             const int kk = k0 + kloc;
-            kvalid = kk < ph.K;
             uint32_t tap, o, th, tw;
-            p.fd_O.divmod(kvalid ? kk : 0, tap, o);
+            p.fd_O.divmod(kk, tap, o);
             ph.fd_ntw.divmod(tap, th, tw);
+            kvalid = (int)th < ph.nth;
             ka_d0 = -(int)th; ka_d1 = -(int)tw;
             ka_off = ((int)o - ((int)th * p.Wo + (int)tw) * p.O) * 4;
             kb_off = ((((ph.rh + p.sh * (int)th) * p.kw + ph.rw + p.sw * (int)tw) * p.C) * p.O + (int)o) * 4;
@@ -582,25 +587,22 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
             if (A_KC)
             {
                 const int lim_h = MODE == MODE_FWD ? p.H : p.Ho, lim_w = MODE == MODE_FWD ? p.W : p.Wo;
-                const bool ok = kvalid && (unsigned)(a_h[q] + ka_d0) < (unsigned)lim_h &&
-                                (unsigned)(a_w[q] + ka_d1) < (unsigned)lim_w;
+                const bool ok = (int)kvalid & (int)((unsigned)(a_h[q] + ka_d0) < (unsigned)lim_h) &
+                                (int)((unsigned)(a_w[q] + ka_d1) < (unsigned)lim_w) & (int)(slab < s_end);
                 off = ok ? a_base[q] + ka_off : OOB;
             }
             else
             {
                 const int kk = k0 + a_krow[q];
-                const bool kin = kk < ph.K;
                 uint32_t b, rem, i, j;
-                p.fd_HoWo.divmod(kin ? kk : 0, b, rem);
+                p.fd_HoWo.divmod(kk, b, rem);
                 p.fd_Wo.divmod(rem, i, j);
                 const int h = (int)i * p.sh, w = (int)j * p.sw;
-                const bool ok = kin && a_mvalid && (unsigned)(h + a_dh) < (unsigned)p.H &&
-                                (unsigned)(w + a_dw) < (unsigned)p.W && (tid + q * NTHREADS) < TA::CHUNKS;
+                const bool ok = (int)((int)b < p.N) & (int)a_mvalid & (int)((unsigned)(h + a_dh) < (unsigned)p.H) &
+                                (int)((unsigned)(w + a_dw) < (unsigned)p.W) & (int)((tid + q * NTHREADS) < TA::CHUNKS) &
+                                (int)(slab < s_end);
                 off = ok ? (((int)b * p.H + h) * p.W + w) * p.C * 4 + a_moff : OOB;
             }
-#ifdef EXP_NO_GLOBAL
-            off = OOB;
-#endif
             ra[q] = buf_load4(ra_src, off);
         }
 #pragma unroll
@@ -608,20 +610,17 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
         {
             int off;
             if (B_KC)
-                off = (kvalid && b_off[q] != OOB) ? b_off[q] + kb_off : OOB;
+                off = ((int)kvalid & (int)(b_off[q] != OOB) & (int)(slab < s_end)) ? b_off[q] + kb_off : OOB;
             else
             {
-                off = b_off[q];  // rows past the end of the contraction lie past the end of the buffer
-                if (b_off[q] != OOB)
-                    b_off[q] += BK * p.ncols * 4;
+                // rows past the end of the contraction lie past the end of the buffer
+                off = slab < s_end ? b_off[q] : OOB;
+                b_off[q] = b_off[q] != OOB ? b_off[q] + BK * p.ncols * 4 : OOB;
             }
-#ifdef EXP_NO_GLOBAL
-            off = OOB;
-#endif
             rb[q] = buf_load4(rb_src, off);
         }
     };
-    auto store_lds = [&](int stage) {
+    auto store_lds = [&](const f32x4* ra, const f32x4* rb, int stage) {
 #pragma unroll
         for (int q = 0; q < NA; ++q)
         {
@@ -646,54 +645,64 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
         }
     };
 
-    if (s_begin < s_end)
-    {
-        load_global(s_begin);
-        store_lds(0);
-        __syncthreads();
-        for (int s = s_begin; s < s_end; ++s)
+    auto multiply = [&](int stage) {
+        float4 fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+            fa[0][a] = TA::frag(lds_a[stage], wm0 + a * 32 + l32, 0, half);
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+            fb[0][b] = TB::frag(lds_b[stage], wn0 + b * 32 + l32, 0, half);
+#pragma unroll
+        for (int kg = 0; kg < BK / 8; ++kg)
         {
-            const int stage = (s - s_begin) & 1;
-            if (s + 1 < s_end)
-                load_global(s + 1);
-            float4 fa[2][TM], fb[2][TN];
-#pragma unroll
-            for (int a = 0; a < TM; ++a)
-                fa[0][a] = TA::frag(lds_a[stage], wm0 + a * 32 + l32, 0, half);
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-                fb[0][b] = TB::frag(lds_b[stage], wn0 + b * 32 + l32, 0, half);
-#pragma unroll
-            for (int kg = 0; kg < BK / 8; ++kg)
+            const int cur = kg & 1;
+            if (kg + 1 < BK / 8)
             {
-                const int cur = kg & 1;
-                if (kg + 1 < BK / 8)
-                {
 #pragma unroll
-                    for (int a = 0; a < TM; ++a)
-                        fa[cur ^ 1][a] = TA::frag(lds_a[stage], wm0 + a * 32 + l32, kg + 1, half);
+                for (int a = 0; a < TM; ++a)
+                    fa[cur ^ 1][a] = TA::frag(lds_a[stage], wm0 + a * 32 + l32, kg + 1, half);
+#pragma unroll
+                for (int b = 0; b < TN; ++b)
+                    fb[cur ^ 1][b] = TB::frag(lds_b[stage], wn0 + b * 32 + l32, kg + 1, half);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int a = 0; a < TM; ++a)
 #pragma unroll
                     for (int b = 0; b < TN; ++b)
-                        fb[cur ^ 1][b] = TB::frag(lds_b[stage], wn0 + b * 32 + l32, kg + 1, half);
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int a = 0; a < TM; ++a)
-#pragma unroll
-                        for (int b = 0; b < TN; ++b)
-                            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                                reinterpret_cast<const float*>(&fa[cur][a])[j],
-                                reinterpret_cast<const float*>(&fb[cur][b])[j], acc[a][b], 0, 0, 0);
-            }
-#ifdef EXP_NO_LDS_STORE
-            if (s + 1 < s_end && ra[0].x == 12345.f)
-#else
-            if (s + 1 < s_end)
-#endif
-                store_lds(stage ^ 1);
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                            reinterpret_cast<const float*>(&fa[cur][a])[j],
+                            reinterpret_cast<const float*>(&fb[cur][b])[j], acc[a][b], 0, 0, 0);
+        }
+    };
+
+    // Software pipeline over pairs of slabs; every load and LDS store inside the loop is
+    // unconditional, which keeps the loop body free of branches.
+    const int nmine = s_end - s_begin;
+    if (nmine > 0)
+    {
+        load_global(ra0, rb0, s_begin);
+        load_global(ra1, rb1, s_begin + 1);
+        store_lds(ra0, rb0, 0);
+        __syncthreads();
+        int s = s_begin;
+        for (int pair = 0; pair < nmine / 2; ++pair, s += 2)
+        {
+            // slab s is in LDS stage 0, slab s+1 in flight in register set 1
+            load_global(ra0, rb0, s + 2);
+            multiply(0);
+            store_lds(ra1, rb1, 1);
+            __syncthreads();
+            // slab s+1 is in LDS stage 1, slab s+2 in flight in register set 0
+            load_global(ra1, rb1, s + 3);
+            multiply(1);
+            store_lds(ra0, rb0, 0);
             __syncthreads();
         }
+        if (nmine & 1)
+            multiply(0);
     }
 
     const bool direct = p.splitk == 1;
@@ -1020,6 +1029,7 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
         f.rh = (f.ph + pad_top) % sh; f.rw = (f.pw + pad_left) % sw;
         f.q0h = (f.ph + pad_top) / sh; f.q0w = (f.pw + pad_left) / sw;
         const int nth = f.rh < kh ? (kh - f.rh + sh - 1) / sh : 0;
+        f.nth = nth;
         f.ntw = f.rw < kw ? (kw - f.rw + sw - 1) / sw : 0;
         f.M = N * f.Hp * f.Wp;
         f.K = nth * f.ntw * O;  // 0 taps: the phase is bias/activation of zero
