@@ -57,6 +57,7 @@ struct ConvParams
     int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
     int ncols;            // GEMM n extent: O (FWD, DK) or C (DX)
     int splitk;
+    int vec_out;          // 16-byte stores allowed (n extent divisible by 4, aligned destination and bias)
     size_t out_elems;
     FastDiv fd_HoWo, fd_Wo, fd_C, fd_O, fd_kw;
     Phase phase[MAX_PHASES];
@@ -239,6 +240,79 @@ struct Tile
     }
 };
 
+// Write-out of a wavefront's accumulators.  The MFMAs are issued with the operands exchanged
+// (filter-side fragment first), so that register r of lane l holds
+//     C[m = l % 32][n = 8*(r/4) + 4*(l/32) + r%4]
+// i.e. every group of 4 registers is 4 consecutive output channels of one row: one 16-byte store.
+// With split-K the raw partial sums go to the scratch arena; otherwise bias and activation are
+// applied here.
+template <int MODE, int TM, int TN>
+__device__ __forceinline__ void write_tile(const ConvParams& p, const Phase& ph, f32x16 (&acc)[TM][TN], int m_base,
+                                           int n_base, int l32, int half)
+{
+    const bool direct = p.splitk == 1;
+    float* dst = direct ? p.out : p.part + (size_t)blockIdx.y * p.out_elems;
+#pragma unroll
+    for (int a = 0; a < TM; ++a)
+    {
+        const int m = m_base + a * 32 + l32;
+        if (m >= ph.M)
+            continue;
+        size_t row_off;
+        if (MODE == MODE_DX)
+        {
+            uint32_t b, rem, hh, ww;
+            ph.fd_HpWp.divmod(m, b, rem);
+            ph.fd_Wp.divmod(rem, hh, ww);
+            row_off = (((size_t)b * p.H + hh * p.sh + ph.ph) * p.W + ww * p.sw + ph.pw) * p.C;
+        }
+        else
+            row_off = (size_t)m * p.ncols;
+#pragma unroll
+        for (int b = 0; b < TN; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                const int n = n_base + b * 32 + 8 * g + 4 * half;
+                float4 v = make_float4(acc[a][b][4 * g], acc[a][b][4 * g + 1], acc[a][b][4 * g + 2], acc[a][b][4 * g + 3]);
+                if (p.vec_out)
+                {
+                    if (n >= p.ncols)
+                        continue;
+                    if (direct)
+                    {
+                        if (p.bias)
+                        {
+                            const float4 bb = *reinterpret_cast<const float4*>(p.bias + n);
+                            v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+                        }
+                        v.x = apply_act(v.x, p.act, p.alpha); v.y = apply_act(v.y, p.act, p.alpha);
+                        v.z = apply_act(v.z, p.act, p.alpha); v.w = apply_act(v.w, p.act, p.alpha);
+                    }
+                    *reinterpret_cast<float4*>(dst + row_off + n) = v;
+                }
+                else
+                {
+                    const float* e = reinterpret_cast<const float*>(&v);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                    {
+                        if (n + q >= p.ncols)
+                            continue;
+                        float w = e[q];
+                        if (direct)
+                        {
+                            if (p.bias)
+                                w += p.bias[n + q];
+                            w = apply_act(w, p.act, p.alpha);
+                        }
+                        dst[row_off + n + q] = w;
+                    }
+                }
+            }
+    }
+}
+
 // BM x BN output tile per workgroup, WGM x WGN wavefronts, each owning (BM/WGM) x (BN/WGN).
 template <int MODE, int BM, int BN, int WGM, int WGN, bool VECA, bool VECB>
 __global__ __launch_bounds__(NTHREADS) void conv_igemm(const ConvParams p)
@@ -361,8 +435,8 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm(const ConvParams p)
 #pragma unroll
                         for (int b = 0; b < TN; ++b)
                             acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                                reinterpret_cast<const float*>(&fa[a])[j],
-                                reinterpret_cast<const float*>(&fb[b])[j], acc[a][b], 0, 0, 0);
+                                reinterpret_cast<const float*>(&fb[b])[j],
+                                reinterpret_cast<const float*>(&fa[a])[j], acc[a][b], 0, 0, 0);
             }
             if (s + 1 < s_end)
                 store_lds(stage ^ 1);
@@ -370,43 +444,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm(const ConvParams p)
         }
     }
 
-    // Epilogue.  Accumulator register r of lane l holds C[m = 8*(r/4) + 4*(l/32) + r%4][n = l%32].
-    const bool direct = p.splitk == 1;
-    float* dst = direct ? p.out : p.part + (size_t)blockIdx.y * p.out_elems;
-#pragma unroll
-    for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-        {
-            const int m = m0 + wm0 + a * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-            if (m >= ph.M)
-                continue;
-            size_t row_off;
-            if (MODE == MODE_DX)
-            {
-                uint32_t b, rem, hh, ww;
-                ph.fd_HpWp.divmod(m, b, rem);
-                ph.fd_Wp.divmod(rem, hh, ww);
-                row_off = (((size_t)b * p.H + hh * p.sh + ph.ph) * p.W + ww * p.sw + ph.pw) * p.C;
-            }
-            else
-                row_off = (size_t)m * p.ncols;
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-            {
-                const int n = n0 + wn0 + b * 32 + l32;
-                if (n >= p.ncols)
-                    continue;
-                float v = acc[a][b][r];
-                if (direct)
-                {
-                    if (p.bias)
-                        v += p.bias[n];
-                    v = apply_act(v, p.act, p.alpha);
-                }
-                dst[row_off + n] = v;
-            }
-        }
+    write_tile<MODE, TM, TN>(p, ph, acc, m0 + wm0, n0 + wn0, l32, half);
 }
 
 // ---- fast path -------------------------------------------------------------------------------------
@@ -673,8 +711,8 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
 #pragma unroll
                     for (int b = 0; b < TN; ++b)
                         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                            reinterpret_cast<const float*>(&fa[cur][a])[j],
-                            reinterpret_cast<const float*>(&fb[cur][b])[j], acc[a][b], 0, 0, 0);
+                            reinterpret_cast<const float*>(&fb[cur][b])[j],
+                            reinterpret_cast<const float*>(&fa[cur][a])[j], acc[a][b], 0, 0, 0);
         }
     };
 
@@ -705,42 +743,7 @@ __global__ __launch_bounds__(NTHREADS) void conv_igemm_fast(const ConvParams p, 
             multiply(0);
     }
 
-    const bool direct = p.splitk == 1;
-    float* dst = direct ? p.out : p.part + (size_t)blockIdx.y * p.out_elems;
-#pragma unroll
-    for (int a = 0; a < TM; ++a)
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-        {
-            const int m = m0 + wm0 + a * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-            if (m >= ph.M)
-                continue;
-            size_t row_off;
-            if (MODE == MODE_DX)
-            {
-                uint32_t b, rem, hh, ww;
-                ph.fd_HpWp.divmod(m, b, rem);
-                ph.fd_Wp.divmod(rem, hh, ww);
-                row_off = (((size_t)b * p.H + hh * p.sh + ph.ph) * p.W + ww * p.sw + ph.pw) * p.C;
-            }
-            else
-                row_off = (size_t)m * p.ncols;
-#pragma unroll
-            for (int b = 0; b < TN; ++b)
-            {
-                const int n = n0 + wn0 + b * 32 + l32;
-                if (n >= p.ncols)
-                    continue;
-                float v = acc[a][b][r];
-                if (direct)
-                {
-                    if (p.bias)
-                        v += p.bias[n];
-                    v = apply_act(v, p.act, p.alpha);
-                }
-                dst[row_off + n] = v;
-            }
-        }
+    write_tile<MODE, TM, TN>(p, ph, acc, m0 + wm0, n0 + wn0, l32, half);
 }
 
 // out[i] = act(bias[i % cols] + sum_s part[s][i]) -- the partial sums are added in split order, so
@@ -885,6 +888,8 @@ inline bool aligned16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 
 template <int MODE>
 int run_igemm(ConvParams& p, int nz, int max_m, bool veca, bool vecb, hipStream_t st, TileCfg cfg)
 {
+    p.vec_out = p.ncols % 4 == 0 && aligned16(p.out) && (!p.part || aligned16(p.part)) && p.out_elems % 4 == 0 &&
+                (!p.bias || aligned16(p.bias));
     const int tiles_m = (max_m + cfg.bm - 1) / cfg.bm;
     const int tiles_n = (p.ncols + cfg.bn - 1) / cfg.bn;
     dim3 grid((unsigned)(tiles_m * tiles_n), (unsigned)p.splitk, (unsigned)nz);
