@@ -793,50 +793,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ p
 
 struct TileCfg { int bm, bn; };
 
-// Optional per-kernel timing: when enabled, every conv_igemm launch is bracketed by two HIP events
-// on its stream and tagged with the kernel instantiation and the algorithmic FLOPs of the operator
-// it belongs to.  dh_profile_read() waits for the events and adds them up per tag.
-struct ProfRecord
-{
-    hipEvent_t e0, e1;
-    int tag;
-    double flops;
-};
-struct ProfTotal
-{
-    char name[96];
-    long launches;
-    double ms, flops;
-};
-bool g_prof_on = false;
-std::vector<ProfRecord> g_prof_pending;
-std::vector<hipEvent_t> g_prof_pool;
-std::vector<ProfTotal> g_prof_totals;
 double g_prof_flops = 0.0;  // algorithmic FLOPs of the operator being launched
-
-int prof_tag(const char* name)
-{
-    for (size_t i = 0; i < g_prof_totals.size(); ++i)
-        if (!strcmp(g_prof_totals[i].name, name))
-            return (int)i;
-    ProfTotal t{};
-    snprintf(t.name, sizeof(t.name), "%s", name);
-    g_prof_totals.push_back(t);
-    return (int)g_prof_totals.size() - 1;
-}
-
-hipEvent_t prof_event()
-{
-    if (!g_prof_pool.empty())
-    {
-        hipEvent_t e = g_prof_pool.back();
-        g_prof_pool.pop_back();
-        return e;
-    }
-    hipEvent_t e = nullptr;
-    (void)hipEventCreate(&e);
-    return e;
-}
 
 // Bytes of the two operand tensors, for the buffer descriptors of the fast path (0 = too large).
 struct OperandBytes { size_t a, b; };
@@ -848,19 +805,15 @@ int launch_cfg(const ConvParams& p, dim3 grid, bool veca, bool vecb, hipStream_t
 {
     const bool fast = veca && vecb && !g_force_generic && g_operand_bytes.a > 0 && g_operand_bytes.b > 0 &&
                       g_operand_bytes.a < (size_t(1) << 31) && g_operand_bytes.b < (size_t(1) << 31);
-    ProfRecord rec{};
-    if (g_prof_on)
+    int prof = -1;
+    if (profiling())
     {
         char name[96];
         snprintf(name, sizeof(name), "conv_igemm<%s,%dx%d,%s%s>", MODE == MODE_FWD ? "fwd" : MODE == MODE_DX ? "dx" : "dk",
                  BM, BN, veca ? "v" : "s", vecb ? "v" : "s");
         if (fast)
             snprintf(name, sizeof(name), "conv_igemm_fast<%s,%dx%d>", MODE == MODE_FWD ? "fwd" : MODE == MODE_DX ? "dx" : "dk", BM, BN);
-        rec.tag = prof_tag(name);
-        rec.flops = g_prof_flops;
-        rec.e0 = prof_event();
-        rec.e1 = prof_event();
-        (void)hipEventRecord(rec.e0, st);
+        prof = prof_begin(name, g_prof_flops, st);
     }
     if (fast)
         hipLaunchKernelGGL((conv_igemm_fast<MODE, BM, BN, WGM, WGN>), grid, dim3(NTHREADS), 0, st, p,
@@ -873,11 +826,7 @@ int launch_cfg(const ConvParams& p, dim3 grid, bool veca, bool vecb, hipStream_t
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, false, true>), grid, dim3(NTHREADS), 0, st, p);
     else
         hipLaunchKernelGGL((conv_igemm<MODE, BM, BN, WGM, WGN, false, false>), grid, dim3(NTHREADS), 0, st, p);
-    if (g_prof_on)
-    {
-        (void)hipEventRecord(rec.e1, st);
-        g_prof_pending.push_back(rec);
-    }
+    prof_end(prof, st);
     DH_LAUNCH_CHECK("conv_igemm launch");
     return 0;
 }
@@ -909,14 +858,18 @@ TileCfg pick_tile(long M, long N)
 }
 
 // Enough workgroups to give every compute unit two, as long as each split keeps >= 8 k-slabs.
+int g_force_splitk = 0;  // tests and tuning: > 0 overrides the choice (still at most one split per k-slab)
+
 int pick_splitk(long wgs, long min_slabs)
 {
+    if (g_force_splitk > 0)
+        return (int)(g_force_splitk < min_slabs ? g_force_splitk : (min_slabs > 0 ? min_slabs : 1));
     const long target = 2L * num_cus();
     if (wgs >= target || min_slabs < 16)
         return 1;
     long s = (target + wgs - 1) / wgs;
     if (s > min_slabs / 8) s = min_slabs / 8;
-    if (s > 64) s = 64;
+    if (s > 256) s = 256;
     return s < 1 ? 1 : (int)s;
 }
 
@@ -1011,6 +964,13 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
     DH_TRY(ensure_init());
     DH_TRY(check_geom("dh_conv2d_dx", N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     if (!dy || !k || !dx) return fail(DH_EINVAL, "dh_conv2d_dx: null tensor");
+    if (!g_force_generic)
+    {
+        const int rc = conv_dx_few_channels(dy, k, dx, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias,
+                                            act, alpha, as_stream(stream));
+        if (rc != 1)
+            return rc;
+    }
     ConvParams p{};
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = dy; p.b_src = k; p.out = dx; p.bias = bias; p.act = act; p.alpha = alpha;
@@ -1112,55 +1072,10 @@ int dh_debug_force_generic_conv(int on)
     return 0;
 }
 
-int dh_profile_enable(int on)
+int dh_debug_force_splitk(int splits)
 {
-    DH_TRY(ensure_init());
-    g_prof_on = on != 0;
-    return 0;
-}
-
-int dh_profile_reset(void)
-{
-    DH_TRY(ensure_init());
-    DH_HIP(hipDeviceSynchronize());
-    for (ProfRecord& r : g_prof_pending)
-    {
-        g_prof_pool.push_back(r.e0);
-        g_prof_pool.push_back(r.e1);
-    }
-    g_prof_pending.clear();
-    g_prof_totals.clear();
-    return 0;
-}
-
-int dh_profile_read(char* buf, size_t buf_len)
-{
-    DH_TRY(ensure_init());
-    for (ProfRecord& r : g_prof_pending)
-    {
-        float ms = 0.f;
-        DH_HIP(hipEventSynchronize(r.e1));
-        DH_HIP(hipEventElapsedTime(&ms, r.e0, r.e1));
-        ProfTotal& t = g_prof_totals[r.tag];
-        t.launches += 1;
-        t.ms += ms;
-        t.flops += r.flops;
-        g_prof_pool.push_back(r.e0);
-        g_prof_pool.push_back(r.e1);
-    }
-    g_prof_pending.clear();
-    size_t used = 0;
-    if (buf && buf_len)
-        buf[0] = 0;
-    for (const ProfTotal& t : g_prof_totals)
-    {
-        if (!buf || used >= buf_len)
-            break;
-        const int w = snprintf(buf + used, buf_len - used, "%s\t%ld\t%.6f\t%.0f\n", t.name, t.launches, t.ms, t.flops);
-        if (w < 0 || (size_t)w >= buf_len - used)
-            return fail(DH_EINVAL, "dh_profile_read: buffer too small");
-        used += (size_t)w;
-    }
+    if (splits < 0) return fail(DH_EINVAL, "dh_debug_force_splitk: negative split count");
+    g_force_splitk = splits;
     return 0;
 }
 

@@ -20,6 +20,19 @@ int ensure_init();
 int workspace(size_t bytes, void** ptr);
 int num_cus();
 
+// Per-kernel timing (see dh_profile_enable): prof_begin records an event on `st` and returns a
+// handle (-1 while timing is off), prof_end records the closing event.  `work` is the algorithmic
+// FLOPs or bytes the launch stands for.
+bool profiling();
+int prof_begin(const char* name, double work, hipStream_t st);
+void prof_end(int handle, hipStream_t st);
+
+// Input gradient onto at most 4 channels on the vector ALUs (conv_small.hip).  Returns 1 when the
+// shape is not one it takes (the caller then runs the implicit GEMM), 0 after a launch, else an error.
+int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw,
+                         int C, int sh, int sw, int pt, int pl, int H, int W, const float* bias, int act,
+                         float alpha, hipStream_t st);
+
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 #define DH_TRY(expr)                                   \

@@ -39,6 +39,7 @@ _SIGS = {
     "dh_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "dh_workspace_reserve": [_sz],
     "dh_debug_force_generic_conv": [_i],
+    "dh_debug_force_splitk": [_i],
     "dh_profile_enable": [_i],
     "dh_profile_reset": [],
     "dh_profile_read": [C.c_char_p, _sz],

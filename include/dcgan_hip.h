@@ -80,6 +80,11 @@ int dh_profile_read(char* buf, size_t buf_len);
  * checks, any channel count or alignment) even where the 16-byte buffer-load kernel applies. */
 int dh_debug_force_generic_conv(int on);
 
+/* Test and tuning hook: splits > 0 makes every convolution cut its contraction into that many
+ * splits (at most one per 16-deep k-slab) instead of choosing by occupancy; 0 restores the choice.
+ * The partial sums are added in split order by a second kernel, so results are reproducible. */
+int dh_debug_force_splitk(int splits);
+
 /* ---- convolutions: fp32 implicit GEMM on MFMA, no im2col buffer ------------------------------ */
 
 /* conv2d forward, optionally with the bias add and activation that follow it fused in.

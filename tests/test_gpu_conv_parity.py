@@ -104,6 +104,72 @@ def test_general_kernel_on_vector_shapes(be, orc, shape):
         be.lib.dh_debug_force_generic_conv(0)
 
 
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (2, 64, 64, 3, 5, 5, 64, 2),     # the generator's last layer / discriminator's first, batch 2
+    (3, 19, 13, 1, 5, 5, 8, 2),      # ragged patches on both axes, one channel
+    (2, 17, 33, 2, 3, 3, 72, 2),     # 72 dy channels: a full 64-channel pass and a partial one
+    (1, 20, 14, 4, 4, 4, 12, 2),     # even filter
+    (2, 11, 16, 3, 5, 3, 16, 3),     # stride 3: nine phases, three passes over the wavefronts
+    (1, 10, 10, 3, 2, 2, 4, 3),      # filter smaller than the stride: phases without any tap
+])
+def test_dx_onto_few_channels(be, orc, shape):
+    """Input gradient onto 1-4 channels (vector-ALU kernel with the dy patch staged in LDS) with a
+    fused bias + tanh, against the oracle and against the implicit-GEMM kernel on the same input."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(23, *shape)
+    bias_c = np.linspace(-0.3, 0.3, C).astype(np.float32)
+    orc.set_threads(8)
+    exp = orc.tanh(orc.bias_add(orc.conv2d_input_grad(dy, k, s, (H, W)), bias_c))
+    got = be.conv2d_input_grad(dy, k, s, (H, W), bias=bias_c, act=A.ACT_TANH)
+    close(got, exp, what="few-channel kernel")
+    be.lib.dh_debug_force_generic_conv(1)
+    try:
+        close(be.conv2d_input_grad(dy, k, s, (H, W), bias=bias_c, act=A.ACT_TANH), exp, what="implicit GEMM")
+    finally:
+        be.lib.dh_debug_force_generic_conv(0)
+
+
+@pytest.mark.parametrize("generic", [0, 1])
+@pytest.mark.parametrize("shape", [(3, 12, 12, 36, 5, 5, 72, 2), (2, 16, 16, 128, 5, 5, 256, 2), (4, 9, 7, 3, 5, 5, 10, 2)])
+def test_forced_split_counts(be, orc, shape, generic):
+    """The contraction cut into 3, 7 and 20 splits on shapes that would not be split by themselves:
+    all within tolerance of the oracle and each repeatable to the bit, for the forward and
+    input-gradient products (bias and activation applied in the reduction) and the filter gradient."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(5, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    bias_c = np.linspace(-0.3, 0.3, C).astype(np.float32)
+    orc.set_threads(8)
+    exp_f = orc.relu_leaky(orc.bias_add(orc.conv2d(x, k, (s, s)), bias), 0.2)
+    exp_x = orc.tanh(orc.bias_add(orc.conv2d_input_grad(dy, k, s, (H, W)), bias_c))
+    exp_k = orc.conv2d_kernel_grad(dy, x, s, pads)
+    be.lib.dh_debug_force_generic_conv(generic)
+    try:
+        for splits in (3, 7, 20):
+            be.lib.dh_debug_force_splitk(splits)
+            for rep in range(2):
+                got_f = be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2)
+                got_x = be.conv2d_input_grad(dy, k, s, (H, W), bias=bias_c, act=A.ACT_TANH)
+                got_k = be.conv2d_kernel_grad(dy, x, s, pads)
+                if rep == 0:
+                    first = (got_f, got_x, got_k)
+                    close(got_f, exp_f, what="fwd splits=%d" % splits)
+                    close(got_x, exp_x, what="dx splits=%d" % splits)
+                    close(got_k, exp_k, scale=max(1.0, float(np.abs(exp_k).max())), what="dk splits=%d" % splits)
+                else:
+                    for a, b in zip(first, (got_f, got_x, got_k)):
+                        np.testing.assert_array_equal(a, b)
+    finally:
+        be.lib.dh_debug_force_splitk(0)
+        be.lib.dh_debug_force_generic_conv(0)
+
+
 def test_dk_is_reproducible(be):
     """Split-K partial sums are reduced in a fixed order: two runs give identical bits."""
     x, k, dy = rand_conv_inputs(3, 8, 16, 16, 128, 5, 5, 256, 2)
