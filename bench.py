@@ -8,9 +8,18 @@ parameters are resident in HBM before the timed region starts; synthetic data, r
 
 Prints ONE JSON line.  Besides the contract fields it carries
   roofline      the dominant convolution kernel: algorithmic FLOP/s (HIP events around every launch
-                of that kernel inside the timed region) against the fp32 MFMA peak
+                of that kernel inside the timed region, on the stream it is launched on) against the
+                fp32 MFMA peak; `kernels` lists every convolution kernel the same way and
+                `hbm_kernels` the memory-bound kernels as algorithmic GB/s against the HBM peak
   cpu_baseline  the reference's own CPU operators (oracle/_ref, RT_MODE=CPU arithmetic) timed on this
                 host on a bounded sample and extrapolated to one iteration by FLOPs per operator class
+
+`--workload layers` instead sweeps the four DCGAN layer shapes (forward, input gradient, filter
+gradient separately; BASELINE.json config 1) at `--batch`, each timed over a sustained run, and
+prints one JSON line with a row per (layer, operator).
+
+After the timed region a plain device-to-device copy of 256 MiB runs four times: under
+`rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its known size calibrates the counters.
 """
 import argparse
 import json
@@ -26,6 +35,14 @@ import __graft_entry__ as ge  # noqa: E402
 
 PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0
+CALIBRATION_COPY_BYTES = 256 << 20
+
+# HBM bytes per launch of the convolution kernels in the batch-64 iteration, from two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; averages over the launches of
+# one kernel symbol), each scaled by the same counter's reading for the calibration copy.  The
+# summaries are kept under profiles/.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {
+}
 
 # DCGAN layers: (H, W, C, O) of the equivalent forward convolution, 5x5, stride 2, SAME
 LAYERS = [(64, 64, 3, 64), (32, 32, 64, 128), (16, 16, 128, 256), (8, 8, 256, 512)]
@@ -98,6 +115,77 @@ def cpu_baseline(batch, budget_s=25.0):
             "gflops": {c: rates[c] / 1e9 for c in rates}}
 
 
+def calibration_copy(A):
+    """A plain copy of known size, for scaling the profiler's memory counters."""
+    n = CALIBRATION_COPY_BYTES // 4
+    src, dst = A.Buf((n,)), A.Buf((n,))
+    lib = A.load()
+    A.check(lib.dh_memset0(src.ptr, CALIBRATION_COPY_BYTES, None))
+    for _ in range(4):
+        A.check(lib.dh_memcpy_d2d(dst.ptr, src.ptr, CALIBRATION_COPY_BYTES, None))
+    A.check(lib.dh_sync())
+
+
+def layer_sweep(args, A):
+    """BASELINE.json config 1: every layer shape, forward / input gradient / filter gradient timed
+    separately.  Each operator first runs for about 60 ms (clocks settle), then is timed for at
+    least 100 ms of back-to-back launches with one pair of HIP events on the launch stream."""
+    lib = A.load()
+    N = args.batch
+    rows = []
+    t = A.Timer()
+    for li, (H, W, C, O) in enumerate(LAYERS):
+        Ho, Wo = H // 2, W // 2
+        rng = np.random.default_rng(li)
+        x = A.Buf.from_numpy(rng.uniform(-1, 1, (N, H, W, C)).astype(np.float32))
+        k = A.Buf.from_numpy((rng.standard_normal((5, 5, C, O)) * 0.02).astype(np.float32))
+        dy = A.Buf.from_numpy(rng.uniform(-1, 1, (N, Ho, Wo, O)).astype(np.float32))
+        y, dx, dk = A.Buf((N, Ho, Wo, O)), A.Buf((N, H, W, C)), A.Buf((5, 5, C, O))
+        ops = {
+            "fwd": lambda: A.check(lib.dh_conv2d_fwd(x.ptr, k.ptr, y.ptr, N, H, W, C, 5, 5, O, 2, 2, 1, 1, Ho, Wo,
+                                                     None, 0, 0.0, None)),
+            "dx": lambda: A.check(lib.dh_conv2d_dx(dy.ptr, k.ptr, dx.ptr, N, Ho, Wo, O, 5, 5, C, 2, 2, 1, 1, H, W,
+                                                   None, 0, 0.0, None)),
+            "dk": lambda: A.check(lib.dh_conv2d_dk(x.ptr, dy.ptr, dk.ptr, N, H, W, C, Ho, Wo, O, 5, 5, 2, 2, 1, 1,
+                                                   None)),
+        }
+        flops = conv_flops(N, (H, W, C, O))
+        for name, fn in ops.items():
+            t.start()
+            for _ in range(3):
+                fn()
+            est = max(t.stop_ms() / 3, 1e-3)
+            for _ in range(int(60 / est) + 1):
+                fn()
+            A.check(lib.dh_sync())
+            reps = max(args.steps, int(100 / est) + 1)
+            t.start()
+            for _ in range(reps):
+                fn()
+            ms = t.stop_ms() / reps
+            tf = flops / (ms * 1e-3) / 1e12
+            rows.append({"layer": "D%d" % li, "x": [N, H, W, C], "k": [5, 5, C, O], "op": name, "launches": reps,
+                         "us": round(ms * 1e3, 2), "tflops": round(tf, 2), "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
+    heavy = [r for r in rows if r["layer"] != "D0"]
+    total_fl = sum(conv_flops(N, LAYERS[int(r["layer"][1])]) for r in heavy)
+    total_s = sum(r["us"] * 1e-6 for r in heavy)
+    tf = total_fl / total_s / 1e12
+    worst = min(heavy, key=lambda r: r["frac"])
+    print(json.dumps({
+        "metric": "conv(_transpose) TFLOP/s as % fp32-MFMA peak (layers D1-D3: forward, input gradient, filter gradient)",
+        "value": round(tf, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(total_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: DCGAN layer sweep, fp32, batch %d, 5x5 stride 2 SAME; one step = the nine "
+                               "operators of layers D1-D3 once each (D0 rows listed, not in value)" % N, "batch": N},
+        "device": A.device_info(),
+        "roofline": {"kernel": "%s %s" % (worst["layer"], worst["op"]), "bound": "mfma", "achieved": worst["tflops"],
+                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": worst["frac"], "traffic": None,
+                     "note": "the slowest of the nine operators; every row is in `layers`"},
+        "layers": rows,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -105,6 +193,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--fusion", type=int, default=1)
+    ap.add_argument("--workload", choices=["iteration", "layers"], default="iteration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -112,6 +201,9 @@ def main():
 
     pkg = ge.load_package()
     A = pkg.hipabi
+    if args.workload == "layers":
+        layer_sweep(args, A)
+        return
     weights, z, x = synthetic(args.batch)
     model = pkg.hostabi.DcganModel(args.batch, seed=1, mode="GPU")
     model.set_fusion(bool(args.fusion))
@@ -139,18 +231,34 @@ def main():
     wall = time.perf_counter() - t0
     A.profile_enable(False)
     rows = A.profile_read()
+
+    # second, untimed pass: every kernel bracketed (the events of ~150 small launches per iteration
+    # would slow the timed region itself, so the memory-bound kernels are measured here)
+    A.profile_reset()
+    A.profile_enable(2)
+    aux_steps = max(1, min(20, args.steps))
+    for _ in range(aux_steps):
+        iteration()
+    model.sync()
+    A.profile_enable(False)
+    aux_rows = A.profile_read()
     d_loss = model.eval("d_loss")[0]
     g_loss = model.eval("g_loss")[0]
 
+    calibration_copy(A)
+
     ms_per_step = wall * 1e3 / args.steps
     work = iteration_flops(args.batch)
+    hbm_rows = [r for r in aux_rows if r["name"].startswith("hbm:")]
+    dense_rows = [r for r in aux_rows if r["name"] == "dense gemm"]
     conv_ms = sum(r["ms"] for r in rows)
     conv_fl = sum(r["flops"] for r in rows)
     dom = max(rows, key=lambda r: r["ms"])
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+    traffic = MEASURED_TRAFFIC_BYTES.get(dom["name"]) if args.batch == 64 else None
     roofline = {
         "kernel": dom["name"], "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic,
         "launches": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 2),
         "flops_per_launch": dom["flops"] / dom["launches"],
         "all_conv_kernels": {"tflops": round(conv_fl / (conv_ms * 1e-3) / 1e12, 3),
@@ -158,6 +266,14 @@ def main():
                              "ms_per_step": round(conv_ms / args.steps, 4)},
         "kernels": [{"name": r["name"], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
                      "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2)} for r in sorted(rows, key=lambda r: -r["ms"])],
+        "hbm_kernels": [{"name": r["name"][4:], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+                         "gbs": round(r["flops"] / (r["ms"] * 1e-3) / 1e9, 1),
+                         "frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "ms_per_step": round(r["ms"] / aux_steps, 4)} for r in sorted(hbm_rows, key=lambda r: -r["ms"])],
+        "dense_gemm": [{"launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+                        "ms_per_step": round(r["ms"] / aux_steps, 4)} for r in dense_rows],
+        "hbm_kernels_note": "measured in %d extra iterations after the timed region, algorithmic bytes / "
+                            "event-bracketed launch time (includes the launch gap)" % aux_steps,
     }
     out = {
         "metric": "DCGAN train iters/sec @bs64 fp32; conv(_transpose) TFLOP/s as % fp32-MFMA peak",

@@ -789,6 +789,45 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ p
     }
 }
 
+// The same for many splits and a small output (filter gradients of thin layers): 16 lanes share one
+// 16-byte piece of the output; lane g adds the splits g, g+16, g+32, ... in that order and the 16
+// sums are then combined by a fixed butterfly, so the result is again independent of timing.
+__global__ __launch_bounds__(256) void splitk_reduce_wide(const float* __restrict__ part, float* __restrict__ out,
+                                                          const float* __restrict__ bias, size_t n, int cols,
+                                                          int splitk, int act, float alpha)
+{
+    const size_t n4 = n / 4;
+    const int g = threadIdx.x & 15;
+    const size_t stride = (size_t)gridDim.x * (blockDim.x / 16);
+    for (size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) / 16; i < n4; i += stride)
+    {
+        float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+        for (int k = g; k < splitk; k += 16)
+        {
+            const float4 t = reinterpret_cast<const float4*>(part + (size_t)k * n)[i];
+            s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+        }
+#pragma unroll
+        for (int w = 8; w > 0; w >>= 1)
+        {
+            s.x += __shfl_xor(s.x, w, 16); s.y += __shfl_xor(s.y, w, 16);
+            s.z += __shfl_xor(s.z, w, 16); s.w += __shfl_xor(s.w, w, 16);
+        }
+        if (g == 0)
+        {
+            if (bias)
+            {
+                const float4 b = *reinterpret_cast<const float4*>(bias + (i * 4) % cols);
+                s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+            }
+            s.x = apply_act(s.x, act, alpha); s.y = apply_act(s.y, act, alpha);
+            s.z = apply_act(s.z, act, alpha); s.w = apply_act(s.w, act, alpha);
+            reinterpret_cast<float4*>(out)[i] = s;
+        }
+    }
+}
+
 // ---- host side -----------------------------------------------------------------------------------
 
 struct TileCfg { int bm, bn; };
@@ -912,7 +951,16 @@ int finish_splitk(const ConvParams& p, hipStream_t st)
     unsigned blocks = (unsigned)((work + 255) / 256);
     if (blocks > 4096) blocks = 4096;
     if (blocks == 0) blocks = 1;
-    if (vec)
+    ProfScope prof("hbm:splitk_reduce (4 B x (splits + 1) per output)", 4.0 * n * (p.splitk + 1), st);
+    if (vec && p.splitk >= 32)
+    {
+        // few outputs per split: spread the splits of one output over 16 lanes
+        size_t wide = (n / 4 * 16 + 255) / 256;
+        if (wide > 4096) wide = 4096;
+        hipLaunchKernelGGL(splitk_reduce_wide, dim3((unsigned)wide), dim3(256), 0, st, p.part, p.out, p.bias, n,
+                           p.ncols, p.splitk, p.act, p.alpha);
+    }
+    else if (vec)
         hipLaunchKernelGGL(splitk_reduce<true>, dim3(blocks), dim3(256), 0, st, p.part, p.out, p.bias, n,
                            p.ncols, p.splitk, p.act, p.alpha);
     else

@@ -96,6 +96,7 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     if (!a || !b || !out) return fail(DH_EINVAL, "%s: null tensor", who);
     if (m > 0x7fffffff || n > 0x7fffffff || p > 0x7fffffff) return fail(DH_EINVAL, "%s: extent too large", who);
     hipStream_t st = as_stream(stream);
+    ProfScope prof("dense gemm", 2.0 * m * n * p, st);
     if (m * p <= 4096 && n >= 512)
         hipLaunchKernelGGL(gemm_block_per_output, dim3((unsigned)(m * p)), dim3(256), 0, st, a, b, bias, out,
                            (int)m, (int)n, (int)p, sai, sak, sbk, sbj);

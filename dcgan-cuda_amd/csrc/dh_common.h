@@ -23,9 +23,22 @@ int num_cus();
 // Per-kernel timing (see dh_profile_enable): prof_begin records an event on `st` and returns a
 // handle (-1 while timing is off), prof_end records the closing event.  `work` is the algorithmic
 // FLOPs or bytes the launch stands for.
-bool profiling();
-int prof_begin(const char* name, double work, hipStream_t st);
+// Level 1 times the convolution kernels only (a few dozen launches per training iteration, so the
+// events barely disturb it); level 2 also times the reductions, dense and element-wise kernels.
+bool profiling(int level = 1);
+int prof_begin(const char* name, double work, hipStream_t st, int level = 1);
 void prof_end(int handle, hipStream_t st);
+// Brackets the launches of one scope.  Memory-bound kernels report algorithmic BYTES as their work
+// and carry the prefix "hbm:" in their name.
+struct ProfScope
+{
+    int handle;
+    hipStream_t st;
+    ProfScope(const char* name, double work, hipStream_t s, int level = 2) : handle(prof_begin(name, work, s, level)), st(s) {}
+    ~ProfScope() { prof_end(handle, st); }
+    ProfScope(const ProfScope&) = delete;
+    ProfScope& operator=(const ProfScope&) = delete;
+};
 
 // Input gradient onto at most 4 channels on the vector ALUs (conv_small.hip).  Returns 1 when the
 // shape is not one it takes (the caller then runs the implicit GEMM), 0 after a launch, else an error.

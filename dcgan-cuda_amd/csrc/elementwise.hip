@@ -93,6 +93,7 @@ int run_map1(const char* who, const float* x, float* out, size_t n, void* stream
     if (n == 0) return 0;
     if (!x || !out) return fail(DH_EINVAL, "%s: null tensor", who);
     const bool vec = aligned16(x) && aligned16(out);
+    ProfScope prof("hbm:unary map (8 B/elem)", 8.0 * n, as_stream(stream));
     hipLaunchKernelGGL(map1<F>, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), x, out, n, vec, f);
     DH_LAUNCH_CHECK(who);
     return 0;
@@ -105,6 +106,7 @@ int run_map2(const char* who, const float* a, const float* b, float* out, size_t
     if (n == 0) return 0;
     if (!a || !b || !out) return fail(DH_EINVAL, "%s: null tensor", who);
     const bool vec = aligned16(a) && aligned16(b) && aligned16(out);
+    ProfScope prof("hbm:binary map (12 B/elem)", 12.0 * n, as_stream(stream));
     hipLaunchKernelGGL(map2<F>, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), a, b, out, n, vec, f);
     DH_LAUNCH_CHECK(who);
     return 0;
@@ -298,6 +300,8 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
         partial = static_cast<float*>(ws);
     }
     dim3 grid(col_tiles, (unsigned)chunks);
+    ProfScope prof(fused ? "hbm:activation gradient + column sums (12 B/elem)" : "hbm:column sums (4 B/elem)",
+                   (fused ? 12.0 : 4.0) * rows * cols, st);
     if (fused)
         hipLaunchKernelGGL(colsum_stage1<true>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
                            (uint32_t)cols, G, rows_per_chunk, g);
@@ -593,6 +597,7 @@ int dh_adam_step(float* p, float* m, float* v, const float* g, float m_decay, fl
     if (n == 0) return 0;
     if (!p || !m || !v || !g) return fail(DH_EINVAL, "dh_adam_step: null tensor");
     const bool vec = aligned16(p) && aligned16(m) && aligned16(v) && aligned16(g);
+    ProfScope prof("hbm:adam_step (28 B/param)", 28.0 * n, as_stream(stream));
     hipLaunchKernelGGL(adam_step_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), p, m, v, g,
                        m_decay, m_gain, v_decay, v_gain, lrt, eps, n, vec);
     DH_LAUNCH_CHECK("dh_adam_step");

@@ -24,7 +24,7 @@ struct ProfTotal
     long launches;
     double ms, work;
 };
-bool g_on = false;
+int g_level = 0;   // 0 off, 1 convolution kernels, 2 every tagged kernel
 std::vector<ProfRecord> g_open;      // begun, not yet ended
 std::vector<ProfRecord> g_pending;   // ended, not yet read
 std::vector<hipEvent_t> g_pool;
@@ -55,11 +55,11 @@ hipEvent_t take_event()
 }
 }  // namespace
 
-bool profiling() { return g_on; }
+bool profiling(int level) { return g_level >= level; }
 
-int prof_begin(const char* name, double work, hipStream_t st)
+int prof_begin(const char* name, double work, hipStream_t st, int level)
 {
-    if (!g_on)
+    if (g_level < level)
         return -1;
     ProfRecord r{};
     r.tag = tag_of(name);
@@ -90,7 +90,7 @@ extern "C" {
 int dh_profile_enable(int on)
 {
     DH_TRY(ensure_init());
-    g_on = on != 0;
+    g_level = on < 0 ? 0 : on;
     return 0;
 }
 

@@ -184,7 +184,8 @@ class Timer:
 
 
 def profile_enable(on):
-    check(load().dh_profile_enable(1 if on else 0))
+    """0/False off, 1/True the convolution kernels, 2 every tagged kernel."""
+    check(load().dh_profile_enable(int(on)))
 
 
 def profile_reset():
@@ -192,7 +193,8 @@ def profile_reset():
 
 
 def profile_read():
-    """[{name, launches, ms, flops}] per convolution-kernel instantiation since the last reset."""
+    """[{name, launches, ms, flops}] per kernel tag since the last reset.  `flops` is the algorithmic
+    work of the launches: FLOPs, or bytes for the tags that start with "hbm:"."""
     buf = C.create_string_buffer(1 << 16)
     check(load().dh_profile_read(buf, len(buf)))
     rows = []

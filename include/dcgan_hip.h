@@ -68,10 +68,13 @@ int dh_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop`
 int dh_workspace_reserve(size_t bytes);
 size_t dh_workspace_bytes(void);
 
-/* Per-kernel timing of the convolution kernels (no counterpart in the reference, whose only timer
- * is the per-run wall clock of src/ops/graph.cu:150-169).  While enabled, every implicit-GEMM
- * launch is bracketed by HIP events on its stream.  dh_profile_read() waits for them and writes one
- * line per kernel instantiation: "name<TAB>launches<TAB>total ms<TAB>total algorithmic FLOPs". */
+/* Per-kernel timing (no counterpart in the reference, whose only timer is the per-run wall clock of
+ * src/ops/graph.cu:150-169).  on = 1 brackets the launches of the convolution kernels by HIP events
+ * on the stream they are launched on; on = 2 also those of the reduction, dense and element-wise
+ * kernels (some 150 launches per training iteration: the events then slow the iteration itself).
+ * dh_profile_read() waits for them and writes one line per kernel tag:
+ * "name<TAB>launches<TAB>total ms<TAB>total algorithmic work", the work being FLOPs, or bytes for
+ * the memory-bound kernels, whose tags start with "hbm:". */
 int dh_profile_enable(int on);
 int dh_profile_reset(void);
 int dh_profile_read(char* buf, size_t buf_len);

@@ -135,7 +135,8 @@ def test_dx_onto_few_channels(be, orc, shape):
 @pytest.mark.parametrize("generic", [0, 1])
 @pytest.mark.parametrize("shape", [(3, 12, 12, 36, 5, 5, 72, 2), (2, 16, 16, 128, 5, 5, 256, 2), (4, 9, 7, 3, 5, 5, 10, 2)])
 def test_forced_split_counts(be, orc, shape, generic):
-    """The contraction cut into 3, 7 and 20 splits on shapes that would not be split by themselves:
+    """The contraction cut into 3, 7, 20 and 40 splits (32 and more take the reduction kernel that
+    spreads the splits of one output over 16 lanes) on shapes that would not be split by themselves:
     all within tolerance of the oracle and each repeatable to the bit, for the forward and
     input-gradient products (bias and activation applied in the reduction) and the filter gradient."""
     import __graft_entry__ as ge
@@ -151,7 +152,7 @@ def test_forced_split_counts(be, orc, shape, generic):
     exp_k = orc.conv2d_kernel_grad(dy, x, s, pads)
     be.lib.dh_debug_force_generic_conv(generic)
     try:
-        for splits in (3, 7, 20):
+        for splits in (3, 7, 20, 40):
             be.lib.dh_debug_force_splitk(splits)
             for rep in range(2):
                 got_f = be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2)
