@@ -1,7 +1,10 @@
 // Dense-layer products of the DCGAN (z -> 4*4*512 and 8192 -> 1, and their gradients): well under
-// 1 % of an iteration's FLOPs, so a compact LDS-tiled FMA kernel with strided operand views covers
-// A*B, tr(A)*B and A*tr(B); tall-skinny products with few outputs and a long contraction (8192 -> 1)
-// use one workgroup per output instead.
+// 1 % of an iteration's FLOPs and all of them thin (a batch of 64 rows, a contraction of 1, 64 or
+// 100, or a single output column), so what matters is latency, not arithmetic:
+//   * gemm_skinny: B has unit stride along its columns and the contraction is short: the A operand
+//     (at most 64 rows x 128) is staged in LDS once, every thread streams one column of B;
+//   * gemm_block_per_output: few outputs and a long contraction (8192 -> 1): one workgroup per output;
+//   * gemm_tiled: everything else, an LDS-tiled FMA kernel with strided operand views.
 //
 // Reference counterparts: src/gpu/matmul.cu:12-86 (one thread per output, no tiling).
 #include "dh_common.h"
@@ -65,6 +68,50 @@ __global__ __launch_bounds__(256) void gemm_tiled(const float* __restrict__ a, c
         }
 }
 
+// C[i,j] = sum_k A(i,k) * B(k,j) (+ bias[j]) for K <= SK_MAXK and B(k,j) = b[k*sbk + j] (unit column
+// stride).  A workgroup owns 64 columns and SK_ROWS rows: thread (tx, ty) accumulates rows
+// ty, ty+4, ... of column j0+tx; B[k][j0+tx] is one coalesced load per k shared by its 16 rows, the A
+// values are LDS broadcasts.
+constexpr int SK_ROWS = 64;
+constexpr int SK_MAXK = 128;
+
+__global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, const float* __restrict__ b,
+                                                   const float* __restrict__ bias, float* __restrict__ out,
+                                                   int M, int K, int P, size_t sai, size_t sak, size_t sbk,
+                                                   size_t out_si, size_t out_sj)
+{
+    __shared__ float la[SK_MAXK][SK_ROWS + 1];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int i0 = blockIdx.y * SK_ROWS, j = blockIdx.x * 64 + tx;
+    for (int e = threadIdx.x; e < K * SK_ROWS; e += 256)
+    {
+        int ia, ka;
+        if (sak == 1) { ka = e % K; ia = e / K; } else { ia = e % SK_ROWS; ka = e / SK_ROWS; }
+        la[ka][ia] = i0 + ia < M ? a[(size_t)(i0 + ia) * sai + (size_t)ka * sak] : 0.f;
+    }
+    __syncthreads();
+    float acc[SK_ROWS / 4] = {};
+    if (j < P)
+    {
+#pragma unroll 4
+        for (int k = 0; k < K; ++k)
+        {
+            const float w = b[(size_t)k * sbk + j];
+#pragma unroll
+            for (int r = 0; r < SK_ROWS / 4; ++r)
+                acc[r] = fmaf(la[k][ty + 4 * r], w, acc[r]);
+        }
+        const float bj = bias ? bias[j] : 0.f;
+#pragma unroll
+        for (int r = 0; r < SK_ROWS / 4; ++r)
+        {
+            const int i = i0 + ty + 4 * r;
+            if (i < M)
+                out[(size_t)i * out_si + (size_t)j * out_sj] = acc[r] + bj;
+        }
+    }
+}
+
 // one workgroup per output element: 256 lanes stride over k, then a fixed LDS tree
 __global__ __launch_bounds__(256) void gemm_block_per_output(const float* __restrict__ a, const float* __restrict__ b,
                                                              const float* __restrict__ bias, float* __restrict__ out,
@@ -75,8 +122,21 @@ __global__ __launch_bounds__(256) void gemm_block_per_output(const float* __rest
     const size_t o = blockIdx.x;
     const int i = (int)(o / P), j = (int)(o % P);
     float s = 0.f;
-    for (int k = threadIdx.x; k < K; k += 256)
-        s += a[(size_t)i * sai + (size_t)k * sak] * b[(size_t)k * sbk + (size_t)j * sbj];
+    const float* ar = a + (size_t)i * sai;
+    const float* bc = b + (size_t)j * sbj;
+    if (sak == 1 && sbk == 1 && K % 4 == 0 && ((reinterpret_cast<uintptr_t>(ar) | reinterpret_cast<uintptr_t>(bc)) & 15) == 0)
+    {
+        // both operands contiguous along k: 16-byte loads
+        for (int k = threadIdx.x * 4; k < K; k += 1024)
+        {
+            const float4 x = *reinterpret_cast<const float4*>(ar + k);
+            const float4 y = *reinterpret_cast<const float4*>(bc + k);
+            s += x.x * y.x + x.y * y.y + x.z * y.z + x.w * y.w;
+        }
+    }
+    else
+        for (int k = threadIdx.x; k < K; k += 256)
+            s += ar[(size_t)k * sak] * bc[(size_t)k * sbk];
     lds[threadIdx.x] = s;
     __syncthreads();
     for (int w = 128; w > 0; w >>= 1)
@@ -97,7 +157,15 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     if (m > 0x7fffffff || n > 0x7fffffff || p > 0x7fffffff) return fail(DH_EINVAL, "%s: extent too large", who);
     hipStream_t st = as_stream(stream);
     ProfScope prof("dense gemm", 2.0 * m * n * p, st);
-    if (m * p <= 4096 && n >= 512)
+    if (n <= SK_MAXK && sbj == 1 && p >= 64)
+        hipLaunchKernelGGL(gemm_skinny, dim3((unsigned)((p + 63) / 64), (unsigned)((m + SK_ROWS - 1) / SK_ROWS)), dim3(256),
+                           0, st, a, b, bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+    else if (n <= SK_MAXK && p == 1 && sai == 1 && !bias && m >= 64)
+        // a single output column: out[i] = sum_k a[k*sak + i] * b[k*sbk] is the row vector b times the
+        // matrix a, whose rows are contiguous -- the same kernel with the roles exchanged
+        hipLaunchKernelGGL(gemm_skinny, dim3((unsigned)((m + 63) / 64), 1u), dim3(256), 0, st, b, a, bias, out, 1, (int)n,
+                           (int)m, (size_t)0, sbk, sak, (size_t)0, (size_t)1);
+    else if (m * p <= 4096 && n >= 512)
         hipLaunchKernelGGL(gemm_block_per_output, dim3((unsigned)(m * p)), dim3(256), 0, st, a, b, bias, out,
                            (int)m, (int)n, (int)p, sai, sak, sbk, sbj);
     else

@@ -92,7 +92,8 @@ def test_argmax_is_exact(be, orc):
         assert be.argmax_acc(y, yh) == orc.argmax_acc(y, yh)
 
 
-@pytest.mark.parametrize("m,n,p", [(64, 100, 8192), (64, 8192, 1), (9, 33, 17), (1, 1, 1), (130, 70, 65)])
+@pytest.mark.parametrize("m,n,p", [(64, 100, 8192), (64, 8192, 1), (9, 33, 17), (1, 1, 1), (130, 70, 65), (64, 128, 200), (3, 5, 64),
+                                   (200, 129, 70)])
 def test_dense(be, orc, m, n, p):
     rng = np.random.default_rng(m + n + p)
     x = rng.uniform(-1, 1, (m, n)).astype(np.float32)
