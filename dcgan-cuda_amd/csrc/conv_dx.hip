@@ -1,0 +1,84 @@
+// Input-gradient / transposed-convolution entry point: dh_conv2d_dx (see conv_igemm.inc for the kernels).
+#include "conv_igemm.inc"
+
+extern "C" {
+
+int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw,
+                 int C, int sh, int sw, int pad_top, int pad_left, int H, int W, const float* bias, int act,
+                 float alpha, void* stream)
+{
+    DH_TRY(ensure_init());
+    DH_TRY(check_geom("dh_conv2d_dx", N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
+    if (!dy || !k || !dx) return fail(DH_EINVAL, "dh_conv2d_dx: null tensor");
+    if (!g_force_generic)
+    {
+        const int rc = conv_dx_few_channels(dy, k, dx, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias,
+                                            act, alpha, as_stream(stream));
+        if (rc != 1)
+            return rc;
+    }
+    ConvParams p{};
+    fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
+    p.a_src = dy; p.b_src = k; p.out = dx; p.bias = bias; p.act = act; p.alpha = alpha;
+    p.ncols = C;
+    p.out_elems = (size_t)N * H * W * C;
+
+    // one dense GEMM per output phase (h mod sh, w mod sw)
+    Phase all[64];
+    const int nph = sh * sw;
+    if (nph > 64) return fail(DH_EINVAL, "dh_conv2d_dx: stride %dx%d not supported", sh, sw);
+    long max_m = 0, min_slabs = 1L << 40, total_tiles_m = 0;
+    int n_live = 0;
+    for (int q = 0; q < nph; ++q)
+    {
+        Phase f{};
+        f.ph = q / sw; f.pw = q % sw;
+        f.Hp = f.ph < H ? (H - f.ph + sh - 1) / sh : 0;
+        f.Wp = f.pw < W ? (W - f.pw + sw - 1) / sw : 0;
+        if (f.Hp == 0 || f.Wp == 0)
+            continue;  // no output pixel in this phase
+        f.rh = (f.ph + pad_top) % sh; f.rw = (f.pw + pad_left) % sw;
+        f.q0h = (f.ph + pad_top) / sh; f.q0w = (f.pw + pad_left) / sw;
+        const int nth = f.rh < kh ? (kh - f.rh + sh - 1) / sh : 0;
+        f.nth = nth;
+        f.ntw = f.rw < kw ? (kw - f.rw + sw - 1) / sw : 0;
+        f.M = N * f.Hp * f.Wp;
+        f.K = nth * f.ntw * O;  // 0 taps: the phase is bias/activation of zero
+        f.fd_HpWp = FastDiv((uint32_t)f.Hp * f.Wp);
+        f.fd_Wp = FastDiv(f.Wp);
+        f.fd_ntw = FastDiv(f.ntw > 0 ? f.ntw : 1);
+        all[n_live++] = f;
+        if (f.M > max_m) max_m = f.M;
+        const long slabs = (f.K + BK - 1) / BK;
+        if (slabs < min_slabs) min_slabs = slabs;
+    }
+    const TileCfg cfg = pick_tile(max_m, C);
+    for (int q = 0; q < n_live; ++q)
+        total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;
+    p.splitk = pick_splitk(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn), min_slabs);
+    if (p.splitk > 1)
+    {
+        void* ws;
+        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws));
+        p.part = static_cast<float*>(ws);
+    }
+    const bool veca = O % 4 == 0 && aligned16(dy);
+    const bool vecb = O % 4 == 0 && aligned16(k);
+    // one launch covers up to MAX_PHASES phases; the operator's FLOPs are split evenly over launches
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C / ((n_live + MAX_PHASES - 1) / MAX_PHASES > 0 ? (n_live + MAX_PHASES - 1) / MAX_PHASES : 1);
+    g_operand_bytes = {(size_t)N * Ho * Wo * O * 4, (size_t)kh * kw * C * O * 4};
+    for (int z0 = 0; z0 < n_live; z0 += MAX_PHASES)
+    {
+        const int nz = n_live - z0 < MAX_PHASES ? n_live - z0 : MAX_PHASES;
+        long mm = 0;
+        for (int q = 0; q < nz; ++q)
+        {
+            p.phase[q] = all[z0 + q];
+            if (p.phase[q].M > mm) mm = p.phase[q].M;
+        }
+        DH_TRY(run_igemm<MODE_DX>(p, nz, (int)mm, veca, vecb, as_stream(stream), cfg));
+    }
+    return finish_splitk(p, as_stream(stream));
+}
+
+}

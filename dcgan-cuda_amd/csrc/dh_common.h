@@ -46,6 +46,10 @@ int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int 
                          int C, int sh, int sw, int pt, int pl, int H, int W, const float* bias, int act,
                          float alpha, hipStream_t st);
 
+// Test and tuning switches (dh_debug_force_generic_conv, dh_debug_force_splitk).
+extern bool g_force_generic;  // route every convolution through the general kernel
+extern int g_force_splitk;    // > 0: this many k splits (at most one per k-slab) instead of the automatic choice
+
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 #define DH_TRY(expr)                                   \

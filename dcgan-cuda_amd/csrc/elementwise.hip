@@ -456,6 +456,77 @@ __global__ __launch_bounds__(TPB) void adam_step_kernel(float* __restrict__ p, f
         adam1(p[i], m[i], v[i], g[i], b1, c1, b2, c2, lrt, eps);
 }
 
+// Several variables in one launch.  Each workgroup owns ADAM_BLOCK consecutive elements of one
+// variable; first_block[i] is the first workgroup of item i (a short scalar search finds the item).
+constexpr int ADAM_MAX_ITEMS = 24;
+constexpr int ADAM_BLOCK = TPB * 16;
+
+struct AdamBatch
+{
+    float* p[ADAM_MAX_ITEMS];
+    float* m[ADAM_MAX_ITEMS];
+    float* v[ADAM_MAX_ITEMS];
+    const float* g1[ADAM_MAX_ITEMS];
+    const float* g2[ADAM_MAX_ITEMS];    // second gradient contribution, or null
+    unsigned long long n[ADAM_MAX_ITEMS];
+    float lrt[ADAM_MAX_ITEMS];
+    unsigned first_block[ADAM_MAX_ITEMS + 1];
+    unsigned char vec[ADAM_MAX_ITEMS];  // every pointer of the item 16-byte aligned
+    int count;
+};
+
+__global__ __launch_bounds__(TPB) void adam_step_multi_kernel(const AdamBatch batch, float b1, float c1, float b2, float c2,
+                                                              float eps)
+{
+    int item = 0;
+    while (item + 1 < batch.count && blockIdx.x >= batch.first_block[item + 1])
+        ++item;
+    float* __restrict__ p = batch.p[item];
+    float* __restrict__ m = batch.m[item];
+    float* __restrict__ v = batch.v[item];
+    const float* __restrict__ g1 = batch.g1[item];
+    const float* __restrict__ g2 = batch.g2[item];
+    const size_t n = batch.n[item];
+    const float lrt = batch.lrt[item];
+    const size_t base = (size_t)(blockIdx.x - batch.first_block[item]) * ADAM_BLOCK;
+    if (batch.vec[item])
+    {
+#pragma unroll
+        for (int it = 0; it < ADAM_BLOCK / (TPB * 4); ++it)
+        {
+            const size_t e = base + ((size_t)it * TPB + threadIdx.x) * 4;
+            if (e + 3 < n)
+            {
+                float4 pp = *reinterpret_cast<float4*>(p + e);
+                float4 mm = *reinterpret_cast<float4*>(m + e);
+                float4 vv = *reinterpret_cast<float4*>(v + e);
+                float4 gg = *reinterpret_cast<const float4*>(g1 + e);
+                if (g2)
+                {
+                    const float4 hh = *reinterpret_cast<const float4*>(g2 + e);
+                    gg.x += hh.x; gg.y += hh.y; gg.z += hh.z; gg.w += hh.w;
+                }
+                adam1(pp.x, mm.x, vv.x, gg.x, b1, c1, b2, c2, lrt, eps);
+                adam1(pp.y, mm.y, vv.y, gg.y, b1, c1, b2, c2, lrt, eps);
+                adam1(pp.z, mm.z, vv.z, gg.z, b1, c1, b2, c2, lrt, eps);
+                adam1(pp.w, mm.w, vv.w, gg.w, b1, c1, b2, c2, lrt, eps);
+                *reinterpret_cast<float4*>(p + e) = pp;
+                *reinterpret_cast<float4*>(m + e) = mm;
+                *reinterpret_cast<float4*>(v + e) = vv;
+            }
+            else
+                for (size_t q = e; q < n && q < e + 4; ++q)
+                    adam1(p[q], m[q], v[q], g2 ? g1[q] + g2[q] : g1[q], b1, c1, b2, c2, lrt, eps);
+        }
+    }
+    else
+    {
+        const size_t end = base + ADAM_BLOCK < n ? base + ADAM_BLOCK : n;
+        for (size_t q = base + threadIdx.x; q < end; q += TPB)
+            adam1(p[q], m[q], v[q], g2 ? g1[q] + g2[q] : g1[q], b1, c1, b2, c2, lrt, eps);
+    }
+}
+
 __global__ __launch_bounds__(TPB) void sgd_update_kernel(float* __restrict__ var, const float* __restrict__ dv,
                                                          const float* __restrict__ coeff, size_t n)
 {
@@ -601,6 +672,46 @@ int dh_adam_step(float* p, float* m, float* v, const float* g, float m_decay, fl
     hipLaunchKernelGGL(adam_step_kernel, dim3(grid_for(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, as_stream(stream), p, m, v, g,
                        m_decay, m_gain, v_decay, v_gain, lrt, eps, n, vec);
     DH_LAUNCH_CHECK("dh_adam_step");
+    return 0;
+}
+
+int dh_adam_step_multi(const dh_adam_item* items, int count, float m_decay, float m_gain, float v_decay,
+                       float v_gain, float eps, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (count < 0 || (count > 0 && !items)) return fail(DH_EINVAL, "dh_adam_step_multi: bad item list");
+    hipStream_t st = as_stream(stream);
+    int at = 0;
+    while (at < count)
+    {
+        AdamBatch batch{};
+        unsigned blocks = 0;
+        double bytes = 0.0;
+        for (; at < count && batch.count < ADAM_MAX_ITEMS; ++at)
+        {
+            const dh_adam_item& it = items[at];
+            if (it.n == 0)
+                continue;
+            if (!it.p || !it.m || !it.v || !it.g1) return fail(DH_EINVAL, "dh_adam_step_multi: null tensor in item %d", at);
+            const size_t nb = (it.n + ADAM_BLOCK - 1) / ADAM_BLOCK;
+            if (nb > 0x7fffffffu - blocks) return fail(DH_EINVAL, "dh_adam_step_multi: too many elements");
+            const int i = batch.count++;
+            batch.p[i] = it.p; batch.m[i] = it.m; batch.v[i] = it.v; batch.g1[i] = it.g1; batch.g2[i] = it.g2;
+            batch.n[i] = it.n; batch.lrt[i] = it.lrt;
+            batch.vec[i] = aligned16(it.p) && aligned16(it.m) && aligned16(it.v) && aligned16(it.g1) &&
+                           (!it.g2 || aligned16(it.g2));
+            batch.first_block[i] = blocks;
+            blocks += (unsigned)nb;
+            bytes += (it.g2 ? 32.0 : 28.0) * it.n;
+        }
+        if (batch.count == 0)
+            continue;
+        batch.first_block[batch.count] = blocks;
+        ProfScope prof("hbm:adam_step_multi (28 B/param, 32 with a second gradient)", bytes, st);
+        hipLaunchKernelGGL(adam_step_multi_kernel, dim3(blocks), dim3(TPB), 0, st, batch, m_decay, m_gain, v_decay, v_gain,
+                           eps);
+        DH_LAUNCH_CHECK("dh_adam_step_multi");
+    }
     return 0;
 }
 

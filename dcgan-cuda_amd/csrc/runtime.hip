@@ -96,6 +96,9 @@ int workspace(size_t bytes, void** ptr)
     return 0;
 }
 
+bool g_force_generic = false;
+int g_force_splitk = 0;
+
 }  // namespace dh
 
 using namespace dh;
@@ -232,6 +235,20 @@ int dh_workspace_reserve(size_t bytes)
 size_t dh_workspace_bytes(void)
 {
     return g_cur >= 0 ? g_dev[g_cur].ws_bytes : 0;
+}
+
+
+int dh_debug_force_generic_conv(int on)
+{
+    g_force_generic = on != 0;
+    return 0;
+}
+
+int dh_debug_force_splitk(int splits)
+{
+    if (splits < 0) return fail(DH_EINVAL, "dh_debug_force_splitk: negative split count");
+    g_force_splitk = splits;
+    return 0;
 }
 
 }

@@ -71,6 +71,7 @@ _SIGS = {
     "dh_moment_update2": [_vp, _vp, _f, _f, _sz, _vp],
     "dh_adam_update": [_vp, _vp, _vp, _f, _f, _sz, _vp],
     "dh_adam_step": [_vp, _vp, _vp, _vp, _f, _f, _f, _f, _f, _f, _sz, _vp],
+    "dh_adam_step_multi": [_vp, _i, _f, _f, _f, _f, _f, _vp],
     "dh_sgd_update": [_vp, _vp, _vp, _sz, _vp],
 }
 _RESTYPES = {"dh_version": C.c_char_p, "dh_last_error": C.c_char_p, "dh_workspace_bytes": _sz}
@@ -162,6 +163,12 @@ def device_info():
     check(load().dh_device_info(name, 256, C.byref(cus), C.byref(khz), C.byref(mem)))
     return {"name": name.value.decode(), "compute_units": cus.value, "clock_khz": khz.value,
             "memory_bytes": mem.value}
+
+
+class AdamItem(C.Structure):
+    """dh_adam_item of include/dcgan_hip.h."""
+    _fields_ = [("p", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("g1", C.c_void_p), ("g2", C.c_void_p),
+                ("n", C.c_size_t), ("lrt", C.c_float)]
 
 
 class Timer:
@@ -439,6 +446,20 @@ class HipBackend:
         check(self.lib.dh_adam_step(dp.ptr, dm.ptr, dv.ptr, dg.ptr, beta1, one - np.float32(beta1), beta2,
                                     one - np.float32(beta2), lrt, eps, dp.size, self.stream))
         return dp.numpy(), dm.numpy(), dv.numpy()
+
+    def adam_step_multi(self, items, beta1, beta2, eps):
+        """items: [(p, m, v, g1, g2 or None, lrt)] -> [(p, m, v)] after one step, all in one launch."""
+        arr = (AdamItem * len(items))()
+        bufs = []
+        for i, (p, m, v, g1, g2, lrt) in enumerate(items):
+            dp, dm, dv, dg = self._up(p, m, v, g1)
+            dh = Buf.from_numpy(g2) if g2 is not None else None
+            bufs.append((dp, dm, dv, dg, dh))
+            arr[i] = AdamItem(dp.ptr, dm.ptr, dv.ptr, dg.ptr, dh.ptr if dh else None, dp.size, lrt)
+        one = np.float32(1)
+        check(self.lib.dh_adam_step_multi(arr, len(items), beta1, one - np.float32(beta1), beta2,
+                                          one - np.float32(beta2), eps, self.stream))
+        return [(b[0].numpy(), b[1].numpy(), b[2].numpy()) for b in bufs]
 
     def vect_update(self, var, dv, coeff):
         dvar, ddv, dc = self._up(var, dv, np.array([coeff], np.float32))

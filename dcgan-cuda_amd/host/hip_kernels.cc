@@ -199,14 +199,16 @@ void k_adam_update(rt::Node* n)
 // A step is either one node run through the table or one fused call standing for several nodes.
 struct Step
 {
-    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM } kind = NODE;
+    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM, ADAM_MULTI } kind = NODE;
     rt::Node* node = nullptr;    // NODE: the node; CONV_EPILOGUE: the conv node; ACT_BIAS_GRAD: the act-grad node
     rt::Node* bias = nullptr;    // CONV_EPILOGUE: the mat_rvect_add node (may be null)
     rt::Node* act = nullptr;     // CONV_EPILOGUE: the activation node (may be null)
     rt::Node* sum = nullptr;     // ACT_BIAS_GRAD: the mat_sum_cols node
     rt::Node* m1 = nullptr;      // ADAM: moment_update, moment_update2; node = adam_update
     rt::Node* m2 = nullptr;
+    rt::Node* add = nullptr;     // ADAM: the `add` node that formed the gradient from two contributions (may be null)
     const dbl_t* act_ref = nullptr;  // ACT_BIAS_GRAD: tensor the activation gradient reads
+    std::vector<Step> group;     // ADAM_MULTI: the ADAM steps issued as one launch
 };
 
 int act_code(const rt::Node* n)
@@ -250,6 +252,72 @@ struct Readers
         return it == by_tensor.end() ? none : it->second;
     }
 };
+
+// Every tensor a step reads or writes.
+void tensors_of(const Step& s, std::unordered_set<const dbl_t*>& out)
+{
+    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+        if (n)
+            for (const dbl_t* t : {(const dbl_t*)n->in1, (const dbl_t*)n->in2, (const dbl_t*)n->in3, (const dbl_t*)n->out1})
+                if (t)
+                    out.insert(t);
+    if (s.act_ref)
+        out.insert(s.act_ref);
+}
+
+// Moves the optimiser steps of a plan to its end and issues them as ONE launch.  A step stays where
+// it is when anything after it touches its variable, its moments or its gradient: executing the list
+// in order must give the same values as before.
+void gather_adam_steps(Plan& plan)
+{
+    std::unordered_set<const dbl_t*> later;   // tensors touched by the steps that follow and stay
+    std::vector<Step> kept, moved;
+    for (auto it = plan.steps.rbegin(); it != plan.steps.rend(); ++it)
+    {
+        bool movable = it->kind == Step::ADAM;
+        if (movable)
+        {
+            std::unordered_set<const dbl_t*> mine;
+            tensors_of(*it, mine);
+            for (const dbl_t* t : mine)
+                if (later.count(t))
+                    movable = false;
+            // two optimiser steps on the same variable keep their order: leave both in place
+            for (const Step& m : moved)
+                if (m.node->out1 == it->node->out1)
+                    movable = false;
+        }
+        if (movable)
+            moved.push_back(*it);
+        else
+        {
+            tensors_of(*it, later);
+            kept.push_back(*it);
+        }
+    }
+    if (moved.size() < 2)
+        return;
+    std::reverse(kept.begin(), kept.end());
+    std::reverse(moved.begin(), moved.end());
+    // one launch per set of hyper-parameters (all variables of an optimiser share them)
+    while (!moved.empty())
+    {
+        Step multi;
+        multi.kind = Step::ADAM_MULTI;
+        multi.node = moved.front().node;
+        std::vector<Step> rest;
+        for (const Step& m : moved)
+        {
+            const Step& f = moved.front();
+            const bool same = m.m1->cons1 == f.m1->cons1 && m.m1->cons2 == f.m1->cons2 && m.m2->cons1 == f.m2->cons1 &&
+                              m.m2->cons2 == f.m2->cons2 && m.node->cons4 == f.node->cons4;
+            (same ? multi.group : rest).push_back(m);
+        }
+        kept.push_back(multi);
+        moved.swap(rest);
+    }
+    plan.steps.swap(kept);
+}
 
 Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<const dbl_t*>& keep, bool fuse)
 {
@@ -381,6 +449,22 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
                 absorbed.insert(m1);
                 absorbed.insert(m2);
                 absorbed.insert(n);
+                // gradient = add(a, b) read by nothing but these two moment updates: summed in the kernel
+                for (rt::Node* q : nodes)
+                    if (q->type == rt::Node::OP_ADD && q->out1 == m1->in1 && !absorbed.count(q) && !keep.count(q->out1) &&
+                        q->len1 == n->len1)
+                    {
+                        const auto& rd = readers.of(q->out1);
+                        bool only_moments = !rd.empty();
+                        for (rt::Node* r : rd)
+                            if (r != m1 && r != m2)
+                                only_moments = false;
+                        if (only_moments)
+                        {
+                            s.add = q;
+                            absorbed.insert(q);
+                        }
+                    }
                 fused_at[n] = s;
             }
         }
@@ -416,6 +500,7 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
         s.act_ref = a == z_alias.end() ? nullptr : a->second;
         plan.steps.push_back(s);
     }
+    gather_adam_steps(plan);
     return plan;
 }
 
@@ -471,8 +556,29 @@ void issue(const Step& s)
     {
         rt::Node* a = s.node;
         const float lrt = adam_advance(a);
-        CK(dh_adam_step(a->out1, s.m1->out1, s.m2->out1, s.m1->in1, s.m1->cons1, s.m1->cons2, s.m2->cons1,
-                        s.m2->cons2, lrt, a->cons4, a->len1, g_stream));
+        if (s.add)
+        {
+            dh_adam_item item{a->out1, s.m1->out1, s.m2->out1, s.add->in1, s.add->in2, a->len1, lrt};
+            CK(dh_adam_step_multi(&item, 1, s.m1->cons1, s.m1->cons2, s.m2->cons1, s.m2->cons2, a->cons4, g_stream));
+        }
+        else
+            CK(dh_adam_step(a->out1, s.m1->out1, s.m2->out1, s.m1->in1, s.m1->cons1, s.m1->cons2, s.m2->cons1,
+                            s.m2->cons2, lrt, a->cons4, a->len1, g_stream));
+        return;
+    }
+    case Step::ADAM_MULTI:
+    {
+        std::vector<dh_adam_item> items;
+        for (const Step& g : s.group)
+        {
+            rt::Node* a = g.node;
+            const float lrt = adam_advance(a);
+            items.push_back(dh_adam_item{a->out1, g.m1->out1, g.m2->out1, g.add ? g.add->in1 : g.m1->in1,
+                                         g.add ? g.add->in2 : nullptr, a->len1, lrt});
+        }
+        const Step& f = s.group.front();
+        CK(dh_adam_step_multi(items.data(), (int)items.size(), f.m1->cons1, f.m1->cons2, f.m2->cons1, f.m2->cons2,
+                              f.node->cons4, g_stream));
         return;
     }
     }

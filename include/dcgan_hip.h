@@ -199,6 +199,24 @@ int dh_adam_update(float* p, const float* m, const float* v, float lrt, float ep
  * (the reference passes beta and 1 - beta, src/api/adam-optimizer.cu:48-49). */
 int dh_adam_step(float* p, float* m, float* v, const float* g, float m_decay, float m_gain,
                  float v_decay, float v_gain, float lrt, float eps, size_t n, void* stream);
+
+/* The same step for several variables in ONE launch (a DCGAN optimiser step updates 10 variables,
+ * most of them bias vectors of a few hundred elements).  Item i uses the gradient g1, or g1 + g2
+ * when g2 is not null: that sum is what the reference forms with a separate `add` node when a
+ * variable receives gradient along two paths (src/ops/graph.cu:295-308, src/cpu/ops.hxx:933-938).
+ * lrt is per item because every variable keeps its own step counter (src/ops/adam-update.cu:45). */
+typedef struct dh_adam_item
+{
+    float* p;
+    float* m;
+    float* v;
+    const float* g1;
+    const float* g2;
+    size_t n;
+    float lrt;
+} dh_adam_item;
+int dh_adam_step_multi(const dh_adam_item* items, int count, float m_decay, float m_gain, float v_decay,
+                       float v_gain, float eps, void* stream);
 /* var += *coeff * dv with coeff a DEVICE scalar.  Replaces gpu::vect_update (src/gpu/update.cu:14-21). */
 int dh_sgd_update(float* var, const float* dv, const float* coeff_device, size_t n, void* stream);
 

@@ -124,3 +124,26 @@ def test_adam(be, orc, n):
     gp, gm, gv = be.adam_step(p, m, v, g, 0.5, 0.999, lrt, 1e-8)
     close(gm, em), close(gv, ev), close(gp, ep)
     close(be.vect_update(p, g, -0.1), orc.vect_update(p, g, -0.1))
+
+
+def test_adam_many_variables_in_one_launch(be, orc):
+    """dh_adam_step_multi == the reference's add + moment_update + moment_update2 + adam_update per
+    variable: sizes from one element to several workgroups, with and without a second gradient,
+    more items than one launch holds, each with its own step size."""
+    rng = np.random.default_rng(77)
+    sizes = [1, 3, 64, 100, 4095, 4096, 4097, 12800, 204801] + [5 + 7 * i for i in range(20)]
+    items, expect = [], []
+    for i, n in enumerate(sizes):
+        p = rng.standard_normal(n).astype(np.float32)
+        g1 = rng.standard_normal(n).astype(np.float32)
+        g2 = rng.standard_normal(n).astype(np.float32) if i % 2 == 0 else None
+        m = rng.standard_normal(n).astype(np.float32) * 0.1
+        v = rng.uniform(0, 1, n).astype(np.float32) * 0.01
+        t, lrt = orc.adam_lrt(i % 5, 2e-4, 0.5, 0.999)
+        g = orc.add(g1, g2) if g2 is not None else g1
+        em, ev = orc.moment_update(m, g, 0.5, 0.5), orc.moment_update2(v, g, 0.999, 0.001)
+        expect.append((orc.adam_apply(p, em, ev, lrt, 1e-8), em, ev))
+        items.append((p, m, v, g1, g2, lrt))
+    got = be.adam_step_multi(items, 0.5, 0.999, 1e-8)
+    for (gp, gm, gv), (ep, em, ev) in zip(got, expect):
+        close(gm, em), close(gv, ev), close(gp, ep)
