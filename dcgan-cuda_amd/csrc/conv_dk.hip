@@ -22,7 +22,7 @@ int dh_conv2d_dk(const float* x, const float* dy, float* dk, int N, int H, int W
     if (p.splitk > 1)
     {
         void* ws;
-        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws));
+        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws, as_stream(stream)));
         p.part = static_cast<float*>(ws);
     }
     const bool veca = C % 4 == 0 && aligned16(x);

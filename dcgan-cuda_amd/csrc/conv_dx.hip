@@ -59,7 +59,7 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
     if (p.splitk > 1)
     {
         void* ws;
-        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws));
+        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws, as_stream(stream)));
         p.part = static_cast<float*>(ws);
     }
     const bool veca = O % 4 == 0 && aligned16(dy);

@@ -16,8 +16,10 @@ int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int fail_hip(hipError_t err, const char* what);
 // Makes sure a device is selected and the library state exists (device 0 by default).
 int ensure_init();
-// Scratch arena of the current device, at least `bytes` large (grows, never shrinks).
-int workspace(size_t bytes, void** ptr);
+// Scratch arena of the current device for launches on `stream`, at least `bytes` large (grows, never
+// shrinks).  Each stream has its own, so that split-K launches on different streams may overlap.
+constexpr int MAX_ARENAS = 8;
+int workspace(size_t bytes, void** ptr, hipStream_t stream);
 int num_cus();
 
 // Per-kernel timing (see dh_profile_enable): prof_begin records an event on `st` and returns a

@@ -296,7 +296,7 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     if (db)
     {
         void* ws;
-        DH_TRY(workspace(chunks * cols * sizeof(float), &ws));
+        DH_TRY(workspace(chunks * cols * sizeof(float), &ws, st));
         partial = static_cast<float*>(ws);
     }
     dim3 grid(col_tiles, (unsigned)chunks);

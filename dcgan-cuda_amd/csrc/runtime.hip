@@ -18,8 +18,10 @@ struct DeviceState
     bool ready = false;
     int device = 0;
     int cus = 0;
-    void* ws = nullptr;
-    size_t ws_bytes = 0;
+    // one scratch arena per stream that asked for one: launches on different streams may overlap
+    struct Arena { hipStream_t stream; void* ptr; size_t bytes; };
+    Arena arena[MAX_ARENAS] = {};
+    int n_arenas = 0;
 };
 
 std::mutex g_mu;
@@ -75,24 +77,35 @@ int num_cus()
     return g_cur >= 0 ? g_dev[g_cur].cus : 256;
 }
 
-int workspace(size_t bytes, void** ptr)
+int workspace(size_t bytes, void** ptr, hipStream_t stream)
 {
     DH_TRY(ensure_init());
     std::lock_guard<std::mutex> lock(g_mu);
     DeviceState& st = g_dev[g_cur];
-    if (bytes > st.ws_bytes)
+    DeviceState::Arena* a = nullptr;
+    for (int i = 0; i < st.n_arenas; ++i)
+        if (st.arena[i].stream == stream)
+            a = &st.arena[i];
+    if (!a)
+    {
+        if (st.n_arenas == MAX_ARENAS)
+            return fail(DH_EINVAL, "scratch arenas exist for %d streams already; no room for another stream", MAX_ARENAS);
+        a = &st.arena[st.n_arenas++];
+        *a = DeviceState::Arena{stream, nullptr, 0};
+    }
+    if (bytes > a->bytes)
     {
         // Work queued on the old arena must drain before it is released.
         DH_HIP(hipDeviceSynchronize());
-        if (st.ws)
-            DH_HIP(hipFree(st.ws));
-        st.ws = nullptr;
-        st.ws_bytes = 0;
+        if (a->ptr)
+            DH_HIP(hipFree(a->ptr));
+        a->ptr = nullptr;
+        a->bytes = 0;
         size_t want = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
-        DH_HIP(hipMalloc(&st.ws, want));
-        st.ws_bytes = want;
+        DH_HIP(hipMalloc(&a->ptr, want));
+        a->bytes = want;
     }
-    *ptr = st.ws;
+    *ptr = a->ptr;
     return 0;
 }
 
@@ -180,7 +193,7 @@ int dh_stream_create(void** stream)
 {
     DH_TRY(ensure_init());
     hipStream_t s;
-    DH_HIP(hipStreamCreate(&s));
+    DH_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
     *stream = s;
     return 0;
 }
@@ -219,6 +232,12 @@ int dh_event_record(void* event, void* stream)
     return 0;
 }
 
+int dh_stream_wait_event(void* stream, void* event)
+{
+    DH_HIP(hipStreamWaitEvent(as_stream(stream), static_cast<hipEvent_t>(event), 0));
+    return 0;
+}
+
 int dh_event_elapsed_ms(void* start, void* stop, float* ms)
 {
     DH_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
@@ -229,12 +248,16 @@ int dh_event_elapsed_ms(void* start, void* stop, float* ms)
 int dh_workspace_reserve(size_t bytes)
 {
     void* p;
-    return workspace(bytes, &p);
+    return workspace(bytes, &p, nullptr);
 }
 
 size_t dh_workspace_bytes(void)
 {
-    return g_cur >= 0 ? g_dev[g_cur].ws_bytes : 0;
+    size_t total = 0;
+    if (g_cur >= 0)
+        for (int i = 0; i < g_dev[g_cur].n_arenas; ++i)
+            total += g_dev[g_cur].arena[i].bytes;
+    return total;
 }
 
 

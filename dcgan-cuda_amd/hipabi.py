@@ -31,6 +31,7 @@ _SIGS = {
     "dh_memset0": [_vp, _sz, _vp],
     "dh_sync": [],
     "dh_stream_create": [C.POINTER(_vp)],
+    "dh_stream_wait_event": [_vp, _vp],
     "dh_stream_destroy": [_vp],
     "dh_stream_sync": [_vp],
     "dh_event_create": [C.POINTER(_vp)],

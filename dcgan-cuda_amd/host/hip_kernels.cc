@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <stdexcept>
@@ -501,6 +502,15 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
         plan.steps.push_back(s);
     }
     gather_adam_steps(plan);
+    if (std::getenv("DCGAN_HIP_PLAN_DUMP"))
+    {
+        // the launches a run turns into, for inspection
+        static const char* kinds[] = {"node", "conv+epilogue", "act-grad+bias-grad", "adam", "adam-multi"};
+        std::fprintf(stderr, "plan of %zu nodes -> %zu steps\n", nodes.size(), plan.steps.size());
+        for (const Step& s : plan.steps)
+            std::fprintf(stderr, "  %-20s %-32s len %zu\n", kinds[s.kind], rt::Node::name_of(s.node->type),
+                         (std::size_t)s.node->len1);
+    }
     return plan;
 }
 

@@ -54,16 +54,20 @@ int dh_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* 
 int dh_memset0(void* ptr, size_t bytes, void* stream);
 /* cudaDeviceSynchronize of src/gpu/runner.cu:16, moved out of the per-node loop. */
 int dh_sync(void);
+/* Streams are created non-blocking: work on them is ordered against the default stream and against
+ * each other only through dh_stream_wait_event (the reference has one stream and no events). */
 int dh_stream_create(void** stream);
 int dh_stream_destroy(void* stream);
 int dh_stream_sync(void* stream);
+int dh_stream_wait_event(void* stream, void* event);
 /* HIP events for timing on the stream the kernels run on. */
 int dh_event_create(void** event);
 int dh_event_destroy(void* event);
 int dh_event_record(void* event, void* stream);
 int dh_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
-/* Split-K partial sums live in a per-device scratch arena that grows on demand; reserving the
- * largest size up front keeps hipMalloc out of the steady state.  (Replaces the 3-4
+/* Split-K partial sums live in a scratch arena per device and stream that grows on demand (at most
+ * 8 streams per device may run kernels that need one); reserving the largest size up front, for the
+ * default stream, keeps hipMalloc out of the steady state; dh_workspace_bytes is the sum over streams.  (Replaces the 3-4
  * cudaMalloc/cudaFree per call of src/gpu/conv2d_gemm.hh:514-553.) */
 int dh_workspace_reserve(size_t bytes);
 size_t dh_workspace_bytes(void);
