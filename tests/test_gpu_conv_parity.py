@@ -132,6 +132,28 @@ def test_dx_onto_few_channels(be, orc, shape):
         be.lib.dh_debug_force_generic_conv(0)
 
 
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (2, 64, 64, 3, 5, 5, 64, 2),     # the discriminator's first layer, batch 2
+    (3, 19, 13, 1, 5, 5, 16, 2),     # ragged tiles on both axes, one channel
+    (2, 70, 37, 2, 3, 3, 48, 2),     # more than one tile along both axes, three blocks of output channels
+    (1, 20, 40, 4, 4, 4, 32, 1),     # stride 1, even filter
+    (2, 11, 50, 3, 5, 3, 16, 3),     # stride 3
+])
+def test_fwd_from_few_channels(be, orc, shape):
+    """Forward convolution from 1-4 input channels (12-byte pixels: the scalar-gather path of the
+    implicit GEMM) with a fused bias + leaky relu and without, against the oracle."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(29, *shape)
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    orc.set_threads(8)
+    exp = orc.relu_leaky(orc.bias_add(orc.conv2d(x, k, (s, s)), bias), 0.2)
+    close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), exp, what="with epilogue")
+    close(be.conv2d(x, k, (s, s)), orc.conv2d(x, k, (s, s)), what="no epilogue")
+
+
 @pytest.mark.parametrize("generic", [0, 1])
 @pytest.mark.parametrize("shape", [(3, 12, 12, 36, 5, 5, 72, 2), (2, 16, 16, 128, 5, 5, 256, 2), (4, 9, 7, 3, 5, 5, 10, 2)])
 def test_forced_split_counts(be, orc, shape, generic):
@@ -190,6 +212,47 @@ def test_adjoint_at_full_batch(be):
     b = np.vdot(k.astype(np.float64), be.conv2d_kernel_grad(dy, x, 2, (3, 3)))
     assert abs(lhs - a) <= 1e-4 * abs(lhs) + 1e-2
     assert abs(lhs - b) <= 1e-4 * abs(lhs) + 1e-2
+
+
+@pytest.mark.parametrize("shape", [
+    (512, 32, 32, 64, 5, 5, 128, 2),    # layer D1 at batch 512: no split-K, 4096 row tiles
+    (512, 8, 8, 256, 5, 5, 512, 2),     # layer D3 at batch 512
+    (4096, 64, 64, 3, 5, 5, 64, 2),     # image layer at batch 4096: the largest tensor is [4096,32,32,64], 1.07 GB
+])
+def test_adjoint_at_large_batches(be, shape):
+    """The batch-512 iteration and the batch-4096 generator: sizes where only properties can be checked.
+    <conv(x,k), dy> = <x, dx(dy,k)> = <k, dk(x,dy)>, each inner product accumulated in float64; the
+    filter gradient (a sum over up to 4 million pixels) additionally against a float64 sum of the
+    same products over a sample of its entries."""
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    rng = np.random.default_rng(N + C)
+    x = rng.uniform(-1, 1, (N, H, W, C)).astype(np.float32)
+    k = (rng.standard_normal((kh, kw, C, O)) * 0.02).astype(np.float32)
+    dy = rng.uniform(-1, 1, (N, H // s, W // s, O)).astype(np.float32)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    y = be.conv2d(x, k, (s, s))
+    lhs = np.vdot(y.astype(np.float64).ravel(), dy.astype(np.float64).ravel())
+    del y
+    dx = be.conv2d_input_grad(dy, k, s, (H, W))
+    a = np.vdot(x.astype(np.float64).ravel(), dx.astype(np.float64).ravel())
+    del dx
+    dk = be.conv2d_kernel_grad(dy, x, s, pads)
+    b = np.vdot(k.astype(np.float64).ravel(), dk.astype(np.float64).ravel())
+    # the three values are sums of ~1e9 products of magnitude <= 0.02..1: compare relative to the
+    # root-sum-square scale of such a sum rather than to the (possibly cancelling) value itself
+    scale = max(abs(lhs), 0.02 * np.sqrt(float(dy.size) * kh * kw * C / 3.0))
+    assert abs(lhs - a) <= 1e-4 * scale, (lhs, a)
+    assert abs(lhs - b) <= 1e-4 * scale, (lhs, b)
+    # direct float64 evaluation of a few filter-gradient entries
+    pt, pl = pads[0] // 2, pads[1] // 2
+    for (di, dj, c, o) in [(0, 0, 0, 0), (kh - 1, kw - 1, C - 1, O - 1), (2, 3, C // 2, O // 3)]:
+        xp = np.zeros((N, H + kh, W + kw), np.float64)
+        xp[:, pt:pt + H, pl:pl + W] = x[:, :, :, c]
+        win = xp[:, di:di + s * (H // s):s, dj:dj + s * (W // s):s]
+        exp = float(np.sum(win * dy[:, :, :, o].astype(np.float64)))
+        tol = 1e-4 * abs(exp) + 1e-5 * np.sqrt(float(N) * (H // s) * (W // s))
+        assert abs(float(dk[di, dj, c, o]) - exp) <= tol, ((di, dj, c, o), float(dk[di, dj, c, o]), exp)
 
 
 def test_bad_arguments_are_rejected(be):
