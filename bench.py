@@ -42,10 +42,10 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # one kernel symbol), each scaled by the same counter's reading for the calibration copy.  The
 # summaries are kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000)
-    "conv_igemm_fast<fwd,128x128>": 78.4e6,
-    "conv_igemm_fast<dx,128x128>": 78.8e6,
-    "conv_igemm_fast<dk,128x128>": 115.8e6,
-    "conv_igemm_fast<dx,128x64>": 34.7e6,
+    "conv_igemm_fast<fwd,128x128>": 78.5e6,
+    "conv_igemm_fast<dx,128x128>": 78.0e6,
+    "conv_igemm_fast<dk,128x128>": 116.1e6,
+    "conv_igemm_fast<dx,128x64>": 34.4e6,
     "conv_igemm<fwd,128x64,sv>": 21.7e6,
     "conv_igemm<dk,128x64,sv>": 25.6e6,
     "dx_few_channels": 27.2e6,
