@@ -9,6 +9,8 @@
 // Reference counterparts: src/gpu/matmul.cu:12-86 (one thread per output, no tiling).
 #include "dh_common.h"
 
+#include <type_traits>
+
 using namespace dh;
 
 namespace
@@ -69,43 +71,103 @@ __global__ __launch_bounds__(256) void gemm_tiled(const float* __restrict__ a, c
 }
 
 // C[i,j] = sum_k A(i,k) * B(k,j) (+ bias[j]) for K <= SK_MAXK and B(k,j) = b[k*sbk + j] (unit column
-// stride).  A workgroup owns 64 columns and SK_ROWS rows: thread (tx, ty) accumulates rows
-// ty, ty+4, ... of column j0+tx; B[k][j0+tx] is one coalesced load per k shared by its 16 rows, the A
-// values are LDS broadcasts.
-constexpr int SK_ROWS = 64;
+// stride).  A workgroup owns 64 columns and 4*RPT rows: wavefront ty accumulates rows
+// ty*RPT .. ty*RPT+RPT-1 of column j0+tx; B[k][j0+tx] is one coalesced load per k shared by those rows
+// (the loop is bound by latency, so loads and LDS reads of four k are issued before their FMAs), the
+// A values are LDS broadcasts read RPT at a time.  RPT = 16 serves a batch of 64 rows, RPT = 1 the products with a
+// single row (a vector times a matrix).
 constexpr int SK_MAXK = 128;
 
+template <int RPT>
 __global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, const float* __restrict__ b,
                                                    const float* __restrict__ bias, float* __restrict__ out,
                                                    int M, int K, int P, size_t sai, size_t sak, size_t sbk,
                                                    size_t out_si, size_t out_sj)
 {
-    __shared__ float la[SK_MAXK][SK_ROWS + 1];
+    constexpr int ROWS = 4 * RPT;
+    constexpr int LD = ROWS + 4;   // keeps 16-byte alignment of a wavefront's rows
+    __shared__ __attribute__((aligned(16))) float la[SK_MAXK * LD];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    const int i0 = blockIdx.y * SK_ROWS, j = blockIdx.x * 64 + tx;
-    for (int e = threadIdx.x; e < K * SK_ROWS; e += 256)
+    const int i0 = blockIdx.y * ROWS, j = blockIdx.x * 64 + tx;
+    // stage the A block: lanes run along whichever index is contiguous in memory; eight loads in flight
+    // per thread (addresses are clamped into the matrix and the value discarded, so that nothing here
+    // turns into a branch around a load)
     {
-        int ia, ka;
-        if (sak == 1) { ka = e % K; ia = e / K; } else { ia = e % SK_ROWS; ka = e / SK_ROWS; }
-        la[ka][ia] = i0 + ia < M ? a[(size_t)(i0 + ia) * sai + (size_t)ka * sak] : 0.f;
+        const bool k_fast = sak == 1;
+        const int fast_n = k_fast ? K : ROWS, slow_n = k_fast ? ROWS : K;
+        const int fast_steps = (fast_n + 63) / 64;
+        const int items = ((slow_n + 3) / 4) * fast_steps;   // (slow index, 64-wide fast segment) pairs of this wavefront
+        for (int it0 = 0; it0 < items; it0 += 8)
+        {
+            float v[8];
+            int dst[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+            {
+                const int it = it0 + u;
+                const int slow = ty + 4 * (it / fast_steps), fast = tx + 64 * (it % fast_steps);
+                const int ia = k_fast ? slow : fast, ka = k_fast ? fast : slow;
+                const bool in_tile = it < items && ia < ROWS && ka < K;
+                const bool in_matrix = in_tile && i0 + ia < M;
+                const size_t off = in_matrix ? (size_t)(i0 + ia) * sai + (size_t)ka * sak : 0;
+                const float x = a[off];
+                v[u] = in_matrix ? x : 0.f;
+                dst[u] = in_tile ? ka * LD + ia : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (dst[u] >= 0)
+                    la[dst[u]] = v[u];
+        }
     }
     __syncthreads();
-    float acc[SK_ROWS / 4] = {};
+    float acc[RPT] = {};
     if (j < P)
     {
-#pragma unroll 4
-        for (int k = 0; k < K; ++k)
-        {
-            const float w = b[(size_t)k * sbk + j];
+        const float* mine = la + ty * RPT;
+        // KB k values at a time: their B loads, then their LDS reads, are all issued before the FMAs
+        auto block = [&](int k, auto kb_tag) {
+            constexpr int KB = decltype(kb_tag)::value;
+            float w[KB];
 #pragma unroll
-            for (int r = 0; r < SK_ROWS / 4; ++r)
-                acc[r] = fmaf(la[k][ty + 4 * r], w, acc[r]);
-        }
+            for (int u = 0; u < KB; ++u)
+                w[u] = b[(size_t)(k + u) * sbk + j];
+            float x[KB][RPT];
+#pragma unroll
+            for (int u = 0; u < KB; ++u)
+            {
+                if (RPT % 4 == 0)
+                {
+#pragma unroll
+                    for (int r = 0; r < RPT; r += 4)
+                    {
+                        const float4 q = *reinterpret_cast<const float4*>(mine + (k + u) * LD + r);
+                        x[u][r] = q.x; x[u][r + 1] = q.y; x[u][r + 2] = q.z; x[u][r + 3] = q.w;
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int r = 0; r < RPT; ++r)
+                        x[u][r] = mine[(k + u) * LD + r];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < KB; ++u)
+#pragma unroll
+                for (int r = 0; r < RPT; ++r)
+                    acc[r] = fmaf(x[u][r], w[u], acc[r]);
+        };
+        int k = 0;
+        for (; k + 4 <= K; k += 4)
+            block(k, std::integral_constant<int, 4>{});
+        for (; k < K; ++k)
+            block(k, std::integral_constant<int, 1>{});
         const float bj = bias ? bias[j] : 0.f;
 #pragma unroll
-        for (int r = 0; r < SK_ROWS / 4; ++r)
+        for (int r = 0; r < RPT; ++r)
         {
-            const int i = i0 + ty + 4 * r;
+            const int i = i0 + ty * RPT + r;
             if (i < M)
                 out[(size_t)i * out_si + (size_t)j * out_sj] = acc[r] + bj;
         }
@@ -157,15 +219,18 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     if (m > 0x7fffffff || n > 0x7fffffff || p > 0x7fffffff) return fail(DH_EINVAL, "%s: extent too large", who);
     hipStream_t st = as_stream(stream);
     ProfScope prof("dense gemm", 2.0 * m * n * p, st);
-    if (n <= SK_MAXK && sbj == 1 && p >= 64)
-        hipLaunchKernelGGL(gemm_skinny, dim3((unsigned)((p + 63) / 64), (unsigned)((m + SK_ROWS - 1) / SK_ROWS)), dim3(256),
-                           0, st, a, b, bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+    if (n <= SK_MAXK && sbj == 1 && p >= 64 && m > 4)
+        hipLaunchKernelGGL(gemm_skinny<16>, dim3((unsigned)((p + 63) / 64), (unsigned)((m + 63) / 64)), dim3(256), 0, st, a, b,
+                           bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+    else if (n <= SK_MAXK && sbj == 1 && p >= 64)
+        hipLaunchKernelGGL(gemm_skinny<1>, dim3((unsigned)((p + 63) / 64), 1u), dim3(256), 0, st, a, b, bias, out, (int)m,
+                           (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
     else if (n <= SK_MAXK && p == 1 && sai == 1 && !bias && m >= 64)
         // a single output column: out[i] = sum_k a[k*sak + i] * b[k*sbk] is the row vector b times the
         // matrix a, whose rows are contiguous -- the same kernel with the roles exchanged
-        hipLaunchKernelGGL(gemm_skinny, dim3((unsigned)((m + 63) / 64), 1u), dim3(256), 0, st, b, a, bias, out, 1, (int)n,
+        hipLaunchKernelGGL(gemm_skinny<1>, dim3((unsigned)((m + 63) / 64), 1u), dim3(256), 0, st, b, a, bias, out, 1, (int)n,
                            (int)m, (size_t)0, sbk, sak, (size_t)0, (size_t)1);
-    else if (m * p <= 4096 && n >= 512)
+    else if (m * p <= 16384 && n >= 512)
         hipLaunchKernelGGL(gemm_block_per_output, dim3((unsigned)(m * p)), dim3(256), 0, st, a, b, bias, out,
                            (int)m, (int)n, (int)p, sai, sak, sbk, sbj);
     else
