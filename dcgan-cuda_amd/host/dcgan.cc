@@ -1,4 +1,5 @@
 #include "dcgan.hh"
+#include "images.hh"
 
 #include <cstring>
 #include <stdexcept>
@@ -342,6 +343,29 @@ int dg_eval(void* model, const char* what, float* host, long* count)
         if (host)
             ops::Graph::instance().run({op}, {}, {host});
     });
+}
+
+int dg_save_vars(void*, const char* path) { return guarded([&] { ops::Graph::instance().save_vars(path); }); }
+int dg_load_vars(void*, const char* path) { return guarded([&] { ops::Graph::instance().load_vars(path); }); }
+int dg_save_state(void*, const char* path) { return guarded([&] { ops::Graph::instance().save_state(path); }); }
+int dg_load_state(void*, const char* path) { return guarded([&] { ops::Graph::instance().load_state(path); }); }
+
+int dg_images_normalize(const unsigned char* pix, long count, float* out)
+{
+    return guarded([&] { images::normalize(pix, (std::size_t)count, out); });
+}
+
+int dg_images_load(const char* dir, long idx_beg, long idx_end, float* out)
+{
+    return guarded([&] {
+        const std::vector<dbl_t> batch = images::load(dir, (std::size_t)idx_beg, (std::size_t)idx_end);
+        std::copy(batch.begin(), batch.end(), out);
+    });
+}
+
+int dg_images_save_samples(const float* data, long width, long height, const char* path)
+{
+    return guarded([&] { images::save_samples(data, (std::size_t)width, (std::size_t)height, path); });
 }
 
 int dg_last_schedule_size(void*)

@@ -67,6 +67,18 @@ int dg_generate(void* model, float* images_host);
 //   "grad:g_loss:<var index>", "grad:d_loss:<var index>", "grad:g_loss:x_fake" (d g_loss / d g_out)
 // Returns the number of elements through *count; host may be NULL to query the size only.
 int dg_eval(void* model, const char* what, float* host, long* count);
+// Trainable variables to / from a file (numpy .npz when the path ends in ".npz"); the whole training
+// state (all variables, Adam moments and step counters) as .npz.  The model argument is unused: the
+// operator graph is a process-wide singleton.
+int dg_save_vars(void* model, const char* path);
+int dg_load_vars(void* model, const char* path);
+int dg_save_state(void* model, const char* path);
+int dg_load_state(void* model, const char* path);
+// Image helpers (host/images.hh): 8-bit pixels to [-1, 1]; images <dir>/<6-digit index>.ppm for
+// idx_beg <= index < idx_end as one normalised batch; width x height generated images as one PPM mosaic.
+int dg_images_normalize(const unsigned char* pix, long count, float* out);
+int dg_images_load(const char* dir, long idx_beg, long idx_end, float* out);
+int dg_images_save_samples(const float* data, long width, long height, const char* path);
 // Number of rt::Node instructions / fused launches of the last run.
 int dg_last_schedule_size(void* model);
 }

@@ -1,4 +1,5 @@
 #include "ops.hh"
+#include "npz.hh"
 
 #include <algorithm>
 #include <cmath>
@@ -305,12 +306,52 @@ Op* Graph::compute_gradient_(Op* out, Op* var)
     return succ->child_grad(vari, succ_grad);
 }
 
+namespace
+{
+bool is_npz(const std::string& path)
+{
+    return path.size() > 4 && path.compare(path.size() - 4, 4, ".npz") == 0;
+}
+
+npz::Array to_array(const std::string& name, Variable* v)
+{
+    npz::Array a;
+    a.name = name;
+    const Shape& sh = v->shape_get();
+    for (std::size_t d = 0; d < sh.ndims(); ++d)
+        a.shape.push_back((std::size_t)sh[d]);
+    a.data.resize((std::size_t)sh.total());
+    v->read(a.data.data());
+    return a;
+}
+
+void from_array(const npz::Array& a, Variable* v, const std::string& path)
+{
+    if (a.data.size() != (std::size_t)v->shape_get().total())
+        throw std::runtime_error("load: '" + a.name + "' in " + path + " has " + std::to_string(a.data.size()) +
+                                 " values, the variable " + std::to_string(v->shape_get().total()));
+    v->write(a.data.data());
+}
+}  // namespace
+
+// `.npz` paths: one float32 array per trainable variable, in creation order, under numpy's positional
+// names arr_0, arr_1, ... (the order-based convention of the reference's tensor files,
+// src/ops/graph.cu:326-361).  Other paths: a `DGV1` header, then per variable the element count and
+// the fp32 data.
 void Graph::save_vars(const std::string& path)
 {
+    auto vars = train_vars_get(nullptr);
+    if (is_npz(path))
+    {
+        std::vector<npz::Array> arrays;
+        for (std::size_t i = 0; i < vars.size(); ++i)
+            arrays.push_back(to_array("arr_" + std::to_string(i), vars[i]));
+        npz::save(path, arrays);
+        return;
+    }
     std::FILE* f = std::fopen(path.c_str(), "wb");
     if (!f)
         throw std::runtime_error("save_vars: cannot open " + path);
-    auto vars = train_vars_get(nullptr);
     const std::uint64_t count = vars.size();
     std::fwrite("DGV1", 1, 4, f);
     std::fwrite(&count, sizeof(count), 1, f);
@@ -327,13 +368,30 @@ void Graph::save_vars(const std::string& path)
 
 void Graph::load_vars(const std::string& path)
 {
+    auto vars = train_vars_get(nullptr);
+    if (is_npz(path))
+    {
+        const std::vector<npz::Array> arrays = npz::load(path);
+        if (arrays.size() != vars.size())
+            throw std::runtime_error("load_vars: " + path + " holds " + std::to_string(arrays.size()) + " arrays, the graph " +
+                                     std::to_string(vars.size()) + " trainable variables");
+        for (std::size_t i = 0; i < vars.size(); ++i)
+        {
+            // by name when the archive uses the positional names, else by position
+            const npz::Array* a = &arrays[i];
+            for (const npz::Array& c : arrays)
+                if (c.name == "arr_" + std::to_string(i))
+                    a = &c;
+            from_array(*a, vars[i], path);
+        }
+        return;
+    }
     std::FILE* f = std::fopen(path.c_str(), "rb");
     if (!f)
         throw std::runtime_error("load_vars: cannot open " + path);
     std::unique_ptr<std::FILE, int (*)(std::FILE*)> guard(f, std::fclose);
     char magic[4];
     std::uint64_t count = 0;
-    auto vars = train_vars_get(nullptr);
     if (std::fread(magic, 1, 4, f) != 4 || std::string(magic, 4) != "DGV1" ||
         std::fread(&count, sizeof(count), 1, f) != 1 || count != vars.size())
         throw std::runtime_error("load_vars: " + path + " does not match this graph's variables");
@@ -347,6 +405,45 @@ void Graph::load_vars(const std::string& path)
             throw std::runtime_error("load_vars: truncated file " + path);
         v->write(host.data());
     }
+}
+
+// Everything a training run needs to continue: all variables (the optimisers' moment estimates are
+// non-trainable variables) as var_0, var_1, ... and the step counters of the Adam operators as
+// adam_t.  The reference saves the trainable variables only, so its optimiser restarts from zero
+// moments after a reload.
+void Graph::save_state(const std::string& path)
+{
+    std::vector<npz::Array> arrays;
+    for (std::size_t i = 0; i < vars_.size(); ++i)
+        arrays.push_back(to_array("var_" + std::to_string(i), vars_[i]));
+    npz::Array t;
+    t.name = "adam_t";
+    t.shape = {counters_.size()};
+    for (const auto& c : counters_)
+        t.data.push_back(*c);
+    arrays.push_back(t);
+    npz::save(path, arrays);
+}
+
+void Graph::load_state(const std::string& path)
+{
+    const std::vector<npz::Array> arrays = npz::load(path);
+    auto find = [&](const std::string& name) -> const npz::Array& {
+        for (const npz::Array& a : arrays)
+            if (a.name == name)
+                return a;
+        throw std::runtime_error("load_state: no array '" + name + "' in " + path);
+    };
+    const npz::Array& t = find("adam_t");
+    if (t.data.size() != counters_.size())
+        throw std::runtime_error("load_state: " + path + " holds " + std::to_string(t.data.size()) +
+                                 " step counters, the graph " + std::to_string(counters_.size()));
+    for (std::size_t i = 0; i < vars_.size(); ++i)
+        from_array(find("var_" + std::to_string(i)), vars_[i], path);
+    if (program_mode() == ProgramMode::GPU && !compiled_ops_.empty())
+        hip::synchronize();   // no run may be reading a counter while it changes
+    for (std::size_t i = 0; i < counters_.size(); ++i)
+        *counters_[i] = t.data[i];
 }
 
 void Graph::exit_graph()
@@ -363,6 +460,7 @@ void Graph::exit_graph()
         delete o;
     ops_.clear();
     vars_.clear();
+    counters_.clear();
     input_shapes_.clear();
     grads_.clear();
     schedules_.clear();
@@ -933,6 +1031,7 @@ AdamUpdate* OpsBuilder::adam_update(Variable* var, Op* m, Op* v, dbl_t learning_
     require(var->shape_get() == m->shape_get(), "var and m must have the same shape");
     require(var->shape_get() == v->shape_get(), "var and v must have the same shape");
     auto t = std::make_shared<dbl_t>(0);
+    G().add_counter(t);
     return make("adam_update", var->shape_get(), {var, m, v}, [var, t, learning_rate, beta1, beta2, eps](Op& op) {
         const CompiledOp &cm = CP(op, 1), &cv = CP(op, 2);
         dbl_t* ptr = var->data_begin();

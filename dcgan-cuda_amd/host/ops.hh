@@ -11,6 +11,7 @@
 #include <functional>
 #include <iosfwd>
 #include <map>
+#include <memory>
 #include <string>
 #include <utility>
 #include <vector>
@@ -155,10 +156,15 @@ public:
     Op* gradient(Op* out, Op* var);
 
     void debug_set(bool debug) { debug_ = debug; }
-    // Trainable variables, in creation order, to / from a file (`DGV1` header, then per variable
-    // the element count and the fp32 data).
+    // Trainable variables, in creation order, to / from a file: numpy's .npz when the path ends in
+    // ".npz" (arrays arr_0, arr_1, ...), else a `DGV1` header followed per variable by the element
+    // count and the fp32 data.
     void save_vars(const std::string& path);
     void load_vars(const std::string& path);
+    // All variables (optimiser moments included) and the Adam step counters, as .npz.
+    void save_state(const std::string& path);
+    void load_state(const std::string& path);
+    void add_counter(std::shared_ptr<dbl_t> t) { counters_.push_back(std::move(t)); }
     // Free every operator, tensor and instruction (end of program, or between tests).
     void exit_graph();
 
@@ -173,6 +179,7 @@ private:
 
     std::vector<Op*> ops_;
     std::vector<Variable*> vars_;
+    std::vector<std::shared_ptr<dbl_t>> counters_;   // step counters of the Adam operators, creation order
     std::map<Input*, Shape> input_shapes_;
     std::map<Op*, CompiledOp> compiled_ops_;
     std::map<std::pair<Op*, Op*>, Op*> grads_;

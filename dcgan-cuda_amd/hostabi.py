@@ -42,6 +42,11 @@ def load():
         lib.dg_generate.argtypes = [C.c_void_p, _fp]
         lib.dg_eval.argtypes = [C.c_void_p, C.c_char_p, _fp, C.POINTER(C.c_long)]
         lib.dg_last_schedule_size.argtypes = [C.c_void_p]
+        for name in ("dg_save_vars", "dg_load_vars", "dg_save_state", "dg_load_state"):
+            getattr(lib, name).argtypes = [C.c_void_p, C.c_char_p]
+        lib.dg_images_normalize.argtypes = [C.c_char_p, C.c_long, _fp]
+        lib.dg_images_load.argtypes = [C.c_char_p, C.c_long, C.c_long, _fp]
+        lib.dg_images_save_samples.argtypes = [_fp, C.c_long, C.c_long, C.c_char_p]
         _lib = lib
     return _lib
 
@@ -152,3 +157,39 @@ class DcganModel:
 
     def last_schedule_size(self):
         return self.lib.dg_last_schedule_size(self.h)
+
+    def save_vars(self, path):
+        """Trainable variables, creation order; numpy .npz (arr_0, arr_1, ...) when path ends in .npz."""
+        _check(self.lib.dg_save_vars(self.h, path.encode()))
+
+    def load_vars(self, path):
+        _check(self.lib.dg_load_vars(self.h, path.encode()))
+
+    def save_state(self, path):
+        """All variables, the Adam moments and step counters (.npz): enough to continue training."""
+        _check(self.lib.dg_save_state(self.h, path.encode()))
+
+    def load_state(self, path):
+        _check(self.lib.dg_load_state(self.h, path.encode()))
+
+
+def images_normalize(pix):
+    """uint8 array -> float32 array of the same shape, pix / 127.5 - 1 (src/datasets/celeba.cu:27-28)."""
+    pix = np.ascontiguousarray(pix, dtype=np.uint8)
+    out = np.empty(pix.shape, np.float32)
+    _check(load().dg_images_normalize(pix.ctypes.data_as(C.c_char_p), pix.size, _p(out)))
+    return out
+
+
+def images_load(directory, idx_beg, idx_end):
+    """<directory>/<6-digit index>.ppm for idx_beg <= index < idx_end -> [n, 64, 64, 3] in [-1, 1]."""
+    out = np.empty((idx_end - idx_beg, 64, 64, 3), np.float32)
+    _check(load().dg_images_load(directory.encode(), idx_beg, idx_end, _p(out)))
+    return out
+
+
+def images_save_samples(data, width, height, path):
+    """width x height images [n, 64, 64, 3] in [-1, 1] -> one PPM mosaic (src/datasets/celeba.cu:44-68)."""
+    data = np.ascontiguousarray(data, dtype=np.float32)
+    assert data.size == width * height * 64 * 64 * 3
+    _check(load().dg_images_save_samples(_p(data), width, height, path.encode()))
