@@ -10,6 +10,13 @@ int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W,
     DH_TRY(ensure_init());
     DH_TRY(check_geom("dh_conv2d_fwd", N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     if (!x || !k || !y) return fail(DH_EINVAL, "dh_conv2d_fwd: null tensor");
+    if (!g_force_generic)
+    {
+        const int rc = conv_fwd_thin(x, k, y, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias, act, alpha,
+                                     as_stream(stream));
+        if (rc != 1)
+            return rc;
+    }
     ConvParams p{};
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = x; p.b_src = k; p.out = y; p.bias = bias; p.act = act; p.alpha = alpha;

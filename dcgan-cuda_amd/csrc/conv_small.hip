@@ -167,10 +167,162 @@ __global__ __launch_bounds__(256) void dx_few_channels(const SmallDxParams p)
     }
 }
 
+// ---- forward from a thin input: contraction of at most 80 ----------------------------------------
+// The discriminator's first layer, [N,64,64,3] -> [N,32,32,64] with a 5x5 filter: the contraction is
+// only kh*kw*C = 75 long and a pixel is 12 bytes, so the tiled kernel spends its time on scalar
+// gathers into LDS.  Here the MFMA operands never pass through LDS: lane (m, h) of a wavefront owns
+// output pixel m of a 32-pixel tile and loads ITS patch values k = h*40 + j straight from global
+// memory into the register that MFMA number j consumes; the filter (at most 80 x 64 values) is
+// staged in LDS once per workgroup and read from there, one value per lane and MFMA.  A wavefront
+// computes TF_TILES tiles.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int TF_KH = 40;           // MFMAs per 32-output-channel block; the contraction is padded to 2 * TF_KH
+constexpr int TF_NB = 2;            // 32-channel blocks: up to 64 output channels
+constexpr int TF_TILES = 1;         // 32-pixel tiles per wavefront
+
+struct ThinFwdParams
+{
+    const float* x;
+    const float* k;
+    float* y;
+    const float* bias;
+    int act;
+    float alpha;
+    int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
+    int K, row;             // kh*kw*C and kw*C (one filter row of taps)
+    int pixels;             // N*Ho*Wo
+    uint32_t x_bytes;
+    FastDiv fd_HoWo, fd_Wo, fd_row, fd_C;
+};
+
+__global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
+{
+    __shared__ float filt[2 * TF_KH * 32 * TF_NB];   // [k][n], zero beyond K and O
+    {
+        // all of a thread's filter loads in flight together (out-of-range elements read element 0 and
+        // are replaced by zero: no branch around a load)
+        constexpr int PER_THREAD = 2 * TF_KH * 32 * TF_NB / 256;
+        float v[PER_THREAD];
+#pragma unroll
+        for (int u = 0; u < PER_THREAD; ++u)
+        {
+            const int e = threadIdx.x + u * 256;
+            const int k = e / (32 * TF_NB), n = e - k * (32 * TF_NB);
+            const bool ok = k < p.K && n < p.O;
+            const float w = p.k[ok ? (size_t)k * p.O + n : 0];
+            v[u] = ok ? w : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < PER_THREAD; ++u)
+            filt[threadIdx.x + u * 256] = v[u];
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const float* bw = filt + half * TF_KH * (32 * TF_NB) + l32;   // + q * 64 + nb * 32
+
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const int tiles = (p.pixels + 31) / 32;
+#pragma unroll 1
+    for (int u = 0; u < TF_TILES; ++u)
+    {
+        const int tile = (blockIdx.x * 4 + wave) * TF_TILES + u;
+        if (tile >= tiles)
+            break;
+        const int pix = tile * 32 + l32;
+        const bool live = pix < p.pixels;
+        uint32_t b, rem, i, j;
+        p.fd_HoWo.divmod(live ? pix : 0, b, rem);
+        p.fd_Wo.divmod(rem, i, j);
+        const int h0 = (int)i * p.sh - p.pt, w0 = (int)j * p.sw - p.pl;
+        const int base = (((int)b * p.H + h0) * p.W + w0) * p.C * 4;
+
+        float a[TF_KH];
+#pragma unroll
+        for (int q = 0; q < TF_KH; ++q)
+        {
+            const int k = half * TF_KH + q;
+            uint32_t di, t, dj, c;
+            p.fd_row.divmod(k, di, t);
+            p.fd_C.divmod(t, dj, c);
+            const bool ok = (int)live & (int)(k < p.K) & (int)((unsigned)(h0 + (int)di) < (unsigned)p.H) &
+                            (int)((unsigned)(w0 + (int)dj) < (unsigned)p.W);
+            const int off = ok ? base + ((int)di * p.W * p.C + (int)t) * 4 : (int)0x80000000u;
+            a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+        }
+        f32x16 acc[TF_NB];
+#pragma unroll
+        for (int nb = 0; nb < TF_NB; ++nb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[nb][r] = 0.f;
+#pragma unroll
+        for (int q = 0; q < TF_KH; ++q)
+#pragma unroll
+            for (int nb = 0; nb < TF_NB; ++nb)
+                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bw[q * (32 * TF_NB) + nb * 32], a[q], acc[nb], 0, 0, 0);
+
+        // register r of lane (m, h) holds channel 32*nb + 8*(r/4) + 4*h + r%4 of pixel m
+        if (live)
+        {
+            float* dst = p.y + (size_t)pix * p.O;
+#pragma unroll
+            for (int nb = 0; nb < TF_NB; ++nb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                {
+                    const int n = nb * 32 + 8 * g + 4 * half;
+                    if (n >= p.O)
+                        continue;
+                    float4 v = make_float4(acc[nb][4 * g], acc[nb][4 * g + 1], acc[nb][4 * g + 2], acc[nb][4 * g + 3]);
+                    if (p.bias)
+                    {
+                        const float4 bb = *reinterpret_cast<const float4*>(p.bias + n);
+                        v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
+                    }
+                    v.x = act_apply(v.x, p.act, p.alpha); v.y = act_apply(v.y, p.act, p.alpha);
+                    v.z = act_apply(v.z, p.act, p.alpha); v.w = act_apply(v.w, p.act, p.alpha);
+                    *reinterpret_cast<float4*>(dst + n) = v;
+                }
+        }
+    }
+}
+
 }  // namespace
 
 namespace dh
 {
+
+// Returns 1 when the shape is not one this kernel takes (the caller then uses the implicit GEMM),
+// 0 after a launch, or an error code.
+int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
+                  int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st)
+{
+    const long K = (long)kh * kw * C;
+    const size_t x_bytes = (size_t)N * H * W * C * 4;
+    if (K > 2 * TF_KH || C > 4 || O > 32 * TF_NB || O % 4 != 0 || x_bytes >= (size_t(1) << 31) ||
+        (reinterpret_cast<uintptr_t>(y) & 15) != 0 || (reinterpret_cast<uintptr_t>(bias) & 15) != 0)
+        return 1;
+    ThinFwdParams p{};
+    p.x = x; p.k = k; p.y = y; p.bias = bias; p.act = act; p.alpha = alpha;
+    p.N = N; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.O = O; p.kh = kh; p.kw = kw;
+    p.sh = sh; p.sw = sw; p.pt = pt; p.pl = pl;
+    p.K = (int)K; p.row = kw * C;
+    p.pixels = N * Ho * Wo;
+    p.x_bytes = (uint32_t)x_bytes;
+    p.fd_HoWo = FastDiv((uint32_t)Ho * Wo); p.fd_Wo = FastDiv(Wo); p.fd_row = FastDiv(kw * C); p.fd_C = FastDiv(C);
+    const long blocks = ((long)(p.pixels + 31) / 32 + 4 * TF_TILES - 1) / (4 * TF_TILES);
+    if (blocks > 0x7fffffffL)
+        return 1;
+    const int prof = prof_begin("fwd_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
+    hipLaunchKernelGGL(fwd_thin, dim3((unsigned)blocks), dim3(256), 0, st, p);
+    prof_end(prof, st);
+    DH_LAUNCH_CHECK("fwd_thin launch");
+    return 0;
+}
+
+
 
 // Returns 1 when the shape is not one this kernel takes (the caller then uses the implicit GEMM),
 // 0 after a launch, or an error code.

@@ -47,6 +47,10 @@ struct ProfScope
 int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw,
                          int C, int sh, int sw, int pt, int pl, int H, int W, const float* bias, int act,
                          float alpha, hipStream_t st);
+// Forward convolution with a contraction of at most 80 (few input channels) and at most 64 output
+// channels, MFMA operands loaded straight from global memory; same return convention.
+int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
+                  int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st);
 
 // Test and tuning switches (dh_debug_force_generic_conv, dh_debug_force_splitk).
 extern bool g_force_generic;  // route every convolution through the general kernel

@@ -138,10 +138,13 @@ def test_dx_onto_few_channels(be, orc, shape):
     (2, 70, 37, 2, 3, 3, 48, 2),     # more than one tile along both axes, three blocks of output channels
     (1, 20, 40, 4, 4, 4, 32, 1),     # stride 1, even filter
     (2, 11, 50, 3, 5, 3, 16, 3),     # stride 3
+    (3, 9, 9, 3, 5, 5, 60, 2),       # 60 output channels: the second 32-channel block is partial
+    (2, 12, 10, 4, 5, 4, 8, 2),      # contraction of exactly 80
 ])
 def test_fwd_from_few_channels(be, orc, shape):
-    """Forward convolution from 1-4 input channels (12-byte pixels: the scalar-gather path of the
-    implicit GEMM) with a fused bias + leaky relu and without, against the oracle."""
+    """Forward convolution from 1-4 input channels with a fused bias + leaky relu and without, against
+    the oracle: through the kernel that loads MFMA operands straight from global memory (contraction
+    of at most 80, at most 64 output channels) and through the implicit GEMM's scalar-gather path."""
     import __graft_entry__ as ge
     A = ge.load_package().hipabi
     print("shape", shape, flush=True)
@@ -152,6 +155,11 @@ def test_fwd_from_few_channels(be, orc, shape):
     exp = orc.relu_leaky(orc.bias_add(orc.conv2d(x, k, (s, s)), bias), 0.2)
     close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), exp, what="with epilogue")
     close(be.conv2d(x, k, (s, s)), orc.conv2d(x, k, (s, s)), what="no epilogue")
+    be.lib.dh_debug_force_generic_conv(1)
+    try:
+        close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), exp, what="implicit GEMM")
+    finally:
+        be.lib.dh_debug_force_generic_conv(0)
 
 
 @pytest.mark.parametrize("generic", [0, 1])
