@@ -1,36 +1,62 @@
-// Filter-gradient entry point: dh_conv2d_dk (see conv_igemm.inc for the kernels).
+// Filter-gradient entry points: dh_conv2d_dk, dh_conv2d_dk_pair (see conv_igemm.inc for the kernels).
 #include "conv_igemm.inc"
 
-extern "C" {
-
-int dh_conv2d_dk(const float* x, const float* dy, float* dk, int N, int H, int W, int C, int Ho, int Wo,
-                 int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left, void* stream)
+namespace
+{
+// dk(x, dy), or dk(x, dy) + dk(x2, dy2) in one contraction over both.
+int conv_dk(const char* who, const float* x, const float* dy, const float* x2, const float* dy2, float* dk, int N, int H,
+            int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left, void* stream)
 {
     DH_TRY(ensure_init());
-    DH_TRY(check_geom("dh_conv2d_dk", N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
-    if (!x || !dy || !dk) return fail(DH_EINVAL, "dh_conv2d_dk: null tensor");
+    DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
+    const bool pair = x2 != nullptr || dy2 != nullptr;
+    if (!x || !dy || !dk || (pair && (!x2 || !dy2))) return fail(DH_EINVAL, "%s: null tensor", who);
     ConvParams p{};
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = x; p.b_src = dy; p.out = dk; p.bias = nullptr; p.act = DH_ACT_NONE; p.alpha = 0.f;
+    p.a_src2 = x2; p.b_src2 = dy2;
     p.ncols = O;
     p.out_elems = (size_t)kh * kw * C * O;
     p.phase[0].M = kh * kw * C;
     p.phase[0].K = N * Ho * Wo;
+    const bool veca = C % 4 == 0 && aligned16(x) && aligned16(x2);
+    const bool vecb = O % 4 == 0 && aligned16(dy) && aligned16(dy2);
+    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)N * Ho * Wo * O * 4};
+    if (pair && !takes_fast_path(veca, vecb))
+        return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
+    const long slabs_one = (p.phase[0].K + BK - 1) / BK;
+    p.pair_slabs = pair ? (int)slabs_one : 0;
     const TileCfg cfg = pick_tile(p.phase[0].M, O);
     const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn);
-    p.splitk = pick_splitk(wgs, (p.phase[0].K + BK - 1) / BK);
+    p.splitk = pick_splitk(wgs, slabs_one * (pair ? 2 : 1));
     if (p.splitk > 1)
     {
         void* ws;
         DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws, as_stream(stream)));
         p.part = static_cast<float*>(ws);
     }
-    const bool veca = C % 4 == 0 && aligned16(x);
-    const bool vecb = O % 4 == 0 && aligned16(dy);
-    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C;
-    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)N * Ho * Wo * O * 4};
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C * (pair ? 2 : 1);
     DH_TRY(run_igemm<MODE_DK>(p, 1, p.phase[0].M, veca, vecb, as_stream(stream), cfg));
     return finish_splitk(p, as_stream(stream));
+}
+}  // namespace
+
+extern "C" {
+
+int dh_conv2d_dk(const float* x, const float* dy, float* dk, int N, int H, int W, int C, int Ho, int Wo,
+                 int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left, void* stream)
+{
+    return conv_dk("dh_conv2d_dk", x, dy, nullptr, nullptr, dk, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left,
+                   stream);
+}
+
+int dh_conv2d_dk_pair(const float* x1, const float* dy1, const float* x2, const float* dy2, float* dk, int N, int H,
+                      int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left,
+                      void* stream)
+{
+    if (!x2 || !dy2) return fail(DH_EINVAL, "dh_conv2d_dk_pair: null tensor");
+    return conv_dk("dh_conv2d_dk_pair", x1, dy1, x2, dy2, dk, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left,
+                   stream);
 }
 
 }

@@ -1,18 +1,21 @@
-// Input-gradient / transposed-convolution entry point: dh_conv2d_dx (see conv_igemm.inc for the kernels).
+// Input-gradient / transposed-convolution entry points: dh_conv2d_dx, dh_conv2d_dx_pair (see
+// conv_igemm.inc for the kernels).
 #include "conv_igemm.inc"
 
 #include <algorithm>
 
-extern "C" {
-
-int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw,
-                 int C, int sh, int sw, int pad_top, int pad_left, int H, int W, const float* bias, int act,
-                 float alpha, void* stream)
+namespace
+{
+// One instance (dy2 == dx2 == nullptr) or two instances that share the filter.
+int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, float* dx, float* dx2, int N, int Ho,
+            int Wo, int O, int kh, int kw, int C, int sh, int sw, int pad_top, int pad_left, int H, int W,
+            const float* bias, int act, float alpha, void* stream)
 {
     DH_TRY(ensure_init());
-    DH_TRY(check_geom("dh_conv2d_dx", N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
-    if (!dy || !k || !dx) return fail(DH_EINVAL, "dh_conv2d_dx: null tensor");
-    if (!g_force_generic)
+    DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
+    const bool pair = dy2 != nullptr || dx2 != nullptr;
+    if (!dy || !k || !dx || (pair && (!dy2 || !dx2))) return fail(DH_EINVAL, "%s: null tensor", who);
+    if (!pair && !g_force_generic)
     {
         const int rc = conv_dx_few_channels(dy, k, dx, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias,
                                             act, alpha, as_stream(stream));
@@ -22,13 +25,14 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
     ConvParams p{};
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = dy; p.b_src = k; p.out = dx; p.bias = bias; p.act = act; p.alpha = alpha;
+    p.a_src2 = dy2; p.out2 = dx2;
     p.ncols = C;
     p.out_elems = (size_t)N * H * W * C;
 
     // one dense GEMM per output phase (h mod sh, w mod sw)
     Phase all[64];
     const int nph = sh * sw;
-    if (nph > 64) return fail(DH_EINVAL, "dh_conv2d_dx: stride %dx%d not supported", sh, sw);
+    if (nph > 64) return fail(DH_EINVAL, "%s: stride %dx%d not supported", who, sh, sw);
     long max_m = 0, min_slabs = 1L << 40, total_tiles_m = 0;
     int n_live = 0;
     for (int q = 0; q < nph; ++q)
@@ -62,21 +66,25 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
     // to +9 points of MFMA peak at batch 64 and 256).
     std::sort(all, all + n_live, [](const Phase& a, const Phase& b) { return a.K > b.K; });
     std::reverse(all + (n_live + 1) / 2, all + n_live);
+    const bool veca = O % 4 == 0 && aligned16(dy) && aligned16(dy2);
+    const bool vecb = O % 4 == 0 && aligned16(k);
+    g_operand_bytes = {(size_t)N * Ho * Wo * O * 4, (size_t)kh * kw * C * O * 4};
+    if (pair && (!takes_fast_path(veca, vecb) || C % 4 != 0))
+        return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
+    const int instances = pair ? 2 : 1;
     const TileCfg cfg = pick_tile(max_m, C);
     for (int q = 0; q < n_live; ++q)
         total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;
-    p.splitk = pick_splitk(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn), min_slabs);
+    p.splitk = pick_splitk(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances, min_slabs);
     if (p.splitk > 1)
     {
         void* ws;
-        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws, as_stream(stream)));
+        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk * instances, &ws, as_stream(stream)));
         p.part = static_cast<float*>(ws);
     }
-    const bool veca = O % 4 == 0 && aligned16(dy);
-    const bool vecb = O % 4 == 0 && aligned16(k);
     // one launch covers up to MAX_PHASES phases; the operator's FLOPs are split evenly over launches
-    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C / ((n_live + MAX_PHASES - 1) / MAX_PHASES > 0 ? (n_live + MAX_PHASES - 1) / MAX_PHASES : 1);
-    g_operand_bytes = {(size_t)N * Ho * Wo * O * 4, (size_t)kh * kw * C * O * 4};
+    const int launches = (n_live + MAX_PHASES - 1) / MAX_PHASES > 0 ? (n_live + MAX_PHASES - 1) / MAX_PHASES : 1;
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C * instances / launches;
     for (int z0 = 0; z0 < n_live; z0 += MAX_PHASES)
     {
         const int nz = n_live - z0 < MAX_PHASES ? n_live - z0 : MAX_PHASES;
@@ -89,6 +97,26 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
         DH_TRY(run_igemm<MODE_DX>(p, nz, (int)mm, veca, vecb, as_stream(stream), cfg));
     }
     return finish_splitk(p, as_stream(stream));
+}
+}  // namespace
+
+extern "C" {
+
+int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw,
+                 int C, int sh, int sw, int pad_top, int pad_left, int H, int W, const float* bias, int act,
+                 float alpha, void* stream)
+{
+    return conv_dx("dh_conv2d_dx", dy, nullptr, k, dx, nullptr, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W,
+                   bias, act, alpha, stream);
+}
+
+int dh_conv2d_dx_pair(const float* dy1, const float* dy2, const float* k, float* dx1, float* dx2, int N, int Ho,
+                      int Wo, int O, int kh, int kw, int C, int sh, int sw, int pad_top, int pad_left, int H, int W,
+                      const float* bias, int act, float alpha, void* stream)
+{
+    if (!dy2 || !dx2) return fail(DH_EINVAL, "dh_conv2d_dx_pair: null tensor");
+    return conv_dx("dh_conv2d_dx_pair", dy1, dy2, k, dx1, dx2, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W,
+                   bias, act, alpha, stream);
 }
 
 }

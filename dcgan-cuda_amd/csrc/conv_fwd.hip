@@ -1,16 +1,18 @@
-// Forward convolution entry point: dh_conv2d_fwd (see conv_igemm.inc for the kernels).
+// Forward convolution entry points: dh_conv2d_fwd, dh_conv2d_fwd_pair (see conv_igemm.inc for the kernels).
 #include "conv_igemm.inc"
 
-extern "C" {
-
-int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw,
-                  int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo, const float* bias,
-                  int act, float alpha, void* stream)
+namespace
+{
+// One instance (x2 == y2 == nullptr) or two instances that share the filter.
+int conv_fwd(const char* who, const float* x, const float* x2, const float* k, float* y, float* y2, int N, int H, int W,
+             int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo, const float* bias,
+             int act, float alpha, void* stream)
 {
     DH_TRY(ensure_init());
-    DH_TRY(check_geom("dh_conv2d_fwd", N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
-    if (!x || !k || !y) return fail(DH_EINVAL, "dh_conv2d_fwd: null tensor");
-    if (!g_force_generic)
+    DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
+    const bool pair = x2 != nullptr || y2 != nullptr;
+    if (!x || !k || !y || (pair && (!x2 || !y2))) return fail(DH_EINVAL, "%s: null tensor", who);
+    if (!pair && !g_force_generic)
     {
         const int rc = conv_fwd_thin(x, k, y, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias, act, alpha,
                                      as_stream(stream));
@@ -20,25 +22,49 @@ int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W,
     ConvParams p{};
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = x; p.b_src = k; p.out = y; p.bias = bias; p.act = act; p.alpha = alpha;
+    p.a_src2 = x2; p.out2 = y2;
     p.ncols = O;
     p.out_elems = (size_t)N * Ho * Wo * O;
     p.phase[0].M = N * Ho * Wo;
     p.phase[0].K = kh * kw * C;
+    const bool veca = C % 4 == 0 && aligned16(x) && aligned16(x2);
+    const bool vecb = O % 4 == 0 && aligned16(k);
+    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)kh * kw * C * O * 4};
+    if (pair && !takes_fast_path(veca, vecb))
+        return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const TileCfg cfg = pick_tile(p.phase[0].M, O);
-    const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn);
+    const int instances = pair ? 2 : 1;
+    const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
     p.splitk = pick_splitk(wgs, (p.phase[0].K + BK - 1) / BK);
     if (p.splitk > 1)
     {
         void* ws;
-        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk, &ws, as_stream(stream)));
+        DH_TRY(workspace(p.out_elems * sizeof(float) * p.splitk * instances, &ws, as_stream(stream)));
         p.part = static_cast<float*>(ws);
     }
-    const bool veca = C % 4 == 0 && aligned16(x);
-    const bool vecb = O % 4 == 0 && aligned16(k);
-    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C;
-    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)kh * kw * C * O * 4};
+    g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C * instances;
     DH_TRY(run_igemm<MODE_FWD>(p, 1, p.phase[0].M, veca, vecb, as_stream(stream), cfg));
     return finish_splitk(p, as_stream(stream));
+}
+}  // namespace
+
+extern "C" {
+
+int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw,
+                  int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo, const float* bias,
+                  int act, float alpha, void* stream)
+{
+    return conv_fwd("dh_conv2d_fwd", x, nullptr, k, y, nullptr, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo,
+                    bias, act, alpha, stream);
+}
+
+int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
+                       int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,
+                       const float* bias, int act, float alpha, void* stream)
+{
+    if (!x2 || !y2) return fail(DH_EINVAL, "dh_conv2d_fwd_pair: null tensor");
+    return conv_fwd("dh_conv2d_fwd_pair", x1, x2, k, y1, y2, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias,
+                    act, alpha, stream);
 }
 
 }

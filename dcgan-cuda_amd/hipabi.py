@@ -47,6 +47,9 @@ _SIGS = {
     "dh_conv2d_fwd": [_vp, _vp, _vp] + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dx": [_vp, _vp, _vp] + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dk": [_vp, _vp, _vp] + [_i] * 13 + [_vp],
+    "dh_conv2d_fwd_pair": [_vp] * 5 + [_i] * 13 + [_vp, _i, _f, _vp],
+    "dh_conv2d_dx_pair": [_vp] * 5 + [_i] * 13 + [_vp, _i, _f, _vp],
+    "dh_conv2d_dk_pair": [_vp] * 5 + [_i] * 13 + [_vp],
     "dh_bias_add": [_vp, _vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad": [_vp, _vp, _sz, _sz, _vp],
     "dh_mat_sum_rows": [_vp, _vp, _sz, _sz, _vp],
@@ -245,6 +248,49 @@ class HipBackend:
                                      pads[0] // 2, pads[1] // 2, Ho, Wo, db.ptr if db else None, act, alpha,
                                      self.stream))
         return y.numpy()
+
+    def conv2d_pair(self, x1, x2, k, strides=(2, 2), bias=None, act=ACT_NONE, alpha=0.0):
+        """conv2d of two inputs of one shape with the same filter, in one launch -> (y1, y2)."""
+        N, H, W, Cc = x1.shape
+        assert x2.shape == x1.shape
+        kh, kw, C2, O = k.shape
+        pads = (same_pad(H, kh, strides[0])[0], same_pad(W, kw, strides[1])[0])
+        Ho, Wo = -(-H // strides[0]), -(-W // strides[1])
+        d1, d2, dk = self._up(x1, x2, k)
+        db = Buf.from_numpy(bias) if bias is not None else None
+        y1, y2 = Buf((N, Ho, Wo, O)), Buf((N, Ho, Wo, O))
+        check(self.lib.dh_conv2d_fwd_pair(d1.ptr, d2.ptr, dk.ptr, y1.ptr, y2.ptr, N, H, W, Cc, kh, kw, O, strides[0],
+                                          strides[1], pads[0] // 2, pads[1] // 2, Ho, Wo, db.ptr if db else None, act,
+                                          alpha, self.stream))
+        return y1.numpy(), y2.numpy()
+
+    def conv2d_input_grad_pair(self, dy1, dy2, k, stride, in_hw, bias=None, act=ACT_NONE, alpha=0.0):
+        """conv2d_input_grad of two gradients of one shape with the same filter, in one launch."""
+        N, Ho, Wo, O = dy1.shape
+        assert dy2.shape == dy1.shape
+        kh, kw, Cc, O2 = k.shape
+        H, W = in_hw
+        pad_h = (Ho - 1) * stride + kh - H
+        pad_w = (Wo - 1) * stride + kw - W
+        d1, d2, dk = self._up(dy1, dy2, k)
+        db = Buf.from_numpy(bias) if bias is not None else None
+        o1, o2 = Buf((N, H, W, Cc)), Buf((N, H, W, Cc))
+        check(self.lib.dh_conv2d_dx_pair(d1.ptr, d2.ptr, dk.ptr, o1.ptr, o2.ptr, N, Ho, Wo, O, kh, kw, Cc, stride,
+                                         stride, pad_h // 2, pad_w // 2, H, W, db.ptr if db else None, act, alpha,
+                                         self.stream))
+        return o1.numpy(), o2.numpy()
+
+    def conv2d_kernel_grad_pair(self, dy1, x1, dy2, x2, stride, pads):
+        """conv2d_kernel_grad(dy1, x1) + conv2d_kernel_grad(dy2, x2) as one contraction."""
+        N, Ho, Wo, O = dy1.shape
+        _, H, W, Cc = x1.shape
+        kh = H + pads[0] - stride * (Ho - 1)
+        kw = W + pads[1] - stride * (Wo - 1)
+        a1, b1, a2, b2 = self._up(x1, dy1, x2, dy2)
+        out = Buf((kh, kw, Cc, O))
+        check(self.lib.dh_conv2d_dk_pair(a1.ptr, b1.ptr, a2.ptr, b2.ptr, out.ptr, N, H, W, Cc, Ho, Wo, O, kh, kw,
+                                         stride, stride, pads[0] // 2, pads[1] // 2, self.stream))
+        return out.numpy()
 
     def conv2d_input_grad(self, dy, k, stride, in_hw, bias=None, act=ACT_NONE, alpha=0.0):
         N, Ho, Wo, O = dy.shape

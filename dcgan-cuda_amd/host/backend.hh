@@ -36,6 +36,13 @@ void run_async(rt::NodesList& tasks);
 // Off by default (DCGAN_HIP_FUSE=1 or set_fusion(true) turns it on).
 void set_fusion(bool on);
 bool fusion();
+// Part of fusion, on by default: two steps of a run that are the same convolution with the same
+// filter on independent activations (the discriminator on the real and on the generated batch) are
+// issued as one paired launch; filter gradients that only meet in a sum become one contraction.
+// Call forget_plans() after changing it.
+void set_pairing(bool on);
+// Number of steps (single or fused launches; a reduction that follows a split launch not counted) the last run issued.
+int last_launch_count();
 
 // Tensors the caller will read after the run: the planner keeps them materialised.
 void set_protected_tensors(const std::vector<const dbl_t*>& tensors);

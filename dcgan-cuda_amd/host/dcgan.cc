@@ -262,6 +262,12 @@ void dg_set_fusion(int fuse)
     hip::forget_plans();
 }
 
+void dg_set_pairing(int on)
+{
+    hip::set_pairing(on != 0);
+    hip::forget_plans();
+}
+
 int dg_num_vars(void* model) { return (int)(M(model).g_vars.size() + M(model).d_vars.size()); }
 
 long dg_var_size(void* model, int index)
@@ -367,6 +373,8 @@ int dg_images_save_samples(const float* data, long width, long height, const cha
 {
     return guarded([&] { images::save_samples(data, (std::size_t)width, (std::size_t)height, path); });
 }
+
+int dg_last_launch_count(void*) { return hip::last_launch_count(); }
 
 int dg_last_schedule_size(void*)
 {

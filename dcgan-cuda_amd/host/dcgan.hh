@@ -47,6 +47,8 @@ void* dg_create(int batch, unsigned long long seed);
 void dg_destroy(void* model);
 // fuse != 0: run fused convolution epilogues, activation+bias gradients and single-pass Adam.
 void dg_set_fusion(int fuse);
+// on != 0 (the default): with fusion, same-filter convolutions of independent towers run as one paired launch.
+void dg_set_pairing(int on);
 // Variables in the order g conv-transpose 1..4 (w,b), g dense (w,b), d conv 0..3 (w,b), d dense (w,b).
 int dg_num_vars(void* model);
 long dg_var_size(void* model, int index);
@@ -81,4 +83,5 @@ int dg_images_load(const char* dir, long idx_beg, long idx_end, float* out);
 int dg_images_save_samples(const float* data, long width, long height, const char* path);
 // Number of rt::Node instructions / fused launches of the last run.
 int dg_last_schedule_size(void* model);
+int dg_last_launch_count(void* model);
 }

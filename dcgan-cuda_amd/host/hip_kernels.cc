@@ -6,6 +6,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -25,6 +26,8 @@ namespace
 
 void* g_stream = nullptr;  // the default stream; every launch of the backend is ordered on it
 int g_fusion = -1;         // -1: not decided yet (reads DCGAN_HIP_FUSE)
+int g_last_launches = 0;    // steps of the plan that ran last
+bool g_pairing = true;     // issue same-filter convolutions of independent towers as one launch (part of fusion)
 
 #define CK(call) hip_check((call), #call)
 
@@ -200,7 +203,7 @@ void k_adam_update(rt::Node* n)
 // A step is either one node run through the table or one fused call standing for several nodes.
 struct Step
 {
-    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM, ADAM_MULTI } kind = NODE;
+    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM, ADAM_MULTI, CONV_PAIR } kind = NODE;
     rt::Node* node = nullptr;    // NODE: the node; CONV_EPILOGUE: the conv node; ACT_BIAS_GRAD: the act-grad node
     rt::Node* bias = nullptr;    // CONV_EPILOGUE: the mat_rvect_add node (may be null)
     rt::Node* act = nullptr;     // CONV_EPILOGUE: the activation node (may be null)
@@ -209,7 +212,8 @@ struct Step
     rt::Node* m2 = nullptr;
     rt::Node* add = nullptr;     // ADAM: the `add` node that formed the gradient from two contributions (may be null)
     const dbl_t* act_ref = nullptr;  // ACT_BIAS_GRAD: tensor the activation gradient reads
-    std::vector<Step> group;     // ADAM_MULTI: the ADAM steps issued as one launch
+    std::vector<Step> group;     // ADAM_MULTI: the ADAM steps issued as one launch; CONV_PAIR: the two convolution steps
+    const dbl_t* grad_sum = nullptr;  // ADAM: gradient tensor that already holds the sum of both contributions
 };
 
 int act_code(const rt::Node* n)
@@ -318,6 +322,260 @@ void gather_adam_steps(Plan& plan)
         moved.swap(rest);
     }
     plan.steps.swap(kept);
+}
+
+// ---- paired convolutions ---------------------------------------------------------------------------
+// The discriminator runs twice per optimiser step, on the real and on the generated batch, with the
+// same filters (dcgan/main.cu:304-307).  Two steps that are the same convolution with the same
+// filter on independent activations are issued as ONE launch (dh_conv2d_*_pair): at batch 64 that
+// halves the number of k splits a launch needs.  Two filter gradients whose sum is all the
+// optimiser reads become one contraction over both.  The plan is re-ordered for this (the towers are
+// interleaved layer by layer); every step still runs after the steps that produce its inputs.
+struct ConvCall
+{
+    int kind = -1;            // 0 forward, 1 input gradient / transpose forward, 2 filter gradient
+    ConvGeom g{};
+    const dbl_t* a = nullptr;     // gathered activations (x, dy, x)
+    const dbl_t* b = nullptr;     // filter (forward, input gradient) or dy (filter gradient)
+    dbl_t* out = nullptr;
+    const dbl_t* bias = nullptr;
+    int act = DH_ACT_NONE;
+    float alpha = 0.f;
+};
+
+bool conv_call_of(const Step& s, ConvCall& c)
+{
+    if (s.kind != Step::NODE && s.kind != Step::CONV_EPILOGUE)
+        return false;
+    if (s.kind == Step::NODE && s.act_ref)
+        return false;
+    const rt::Node* n = s.node;
+    switch (n->type)
+    {
+    case rt::Node::OP_CONV2D: c.kind = 0; c.g = geom_conv2d(n); c.a = n->in1; c.b = n->in2; break;
+    case rt::Node::OP_CONV2D_TRANSPOSE_INPUT_GRAD: c.kind = 0; c.g = geom_transpose_input_grad(n); c.a = n->in1; c.b = n->in2; break;
+    case rt::Node::OP_CONV2D_INPUT_GRAD: c.kind = 1; c.g = geom_input_grad(n); c.a = n->in1; c.b = n->in2; break;
+    case rt::Node::OP_CONV2D_TRANSPOSE: c.kind = 1; c.g = geom_transpose(n); c.a = n->in1; c.b = n->in2; break;
+    case rt::Node::OP_CONV2D_KERNEL_GRAD: c.kind = 2; c.g = geom_kernel_grad(n); c.a = n->in2; c.b = n->in1; break;
+    case rt::Node::OP_CONV2D_TRANSPOSE_KERNEL_GRAD: c.kind = 2; c.g = geom_transpose_kernel_grad(n); c.a = n->in1; c.b = n->in2; break;
+    default: return false;
+    }
+    c.out = n->out1;
+    if (s.kind == Step::CONV_EPILOGUE)
+    {
+        if (c.kind == 2)
+            return false;
+        c.bias = s.bias ? s.bias->in2 : nullptr;
+        c.act = s.act ? act_code(s.act) : DH_ACT_NONE;
+        c.alpha = s.act ? s.act->alpha_leaky : 0.f;
+        c.out = s.act ? s.act->out1 : s.bias->out1;
+    }
+    return true;
+}
+
+// What dh_conv2d_*_pair accepts: 16-byte chunks everywhere and operands below 2 GiB.
+bool pairable(const ConvCall& c)
+{
+    const ConvGeom& g = c.g;
+    auto aligned = [](const void* q) { return (reinterpret_cast<std::uintptr_t>(q) & 15) == 0; };
+    const double in_bytes = 4.0 * g.N * g.H * g.W * g.C, out_bytes = 4.0 * g.N * g.Ho * g.Wo * g.O;
+    const double k_bytes = 4.0 * g.kh * g.kw * g.C * g.O, lim = 2147483648.0;
+    return g.C % 4 == 0 && g.O % 4 == 0 && in_bytes < lim && out_bytes < lim && k_bytes < lim && aligned(c.a) &&
+           aligned(c.b) && aligned(c.out) && aligned(c.bias);
+}
+
+bool same_call(const ConvCall& x, const ConvCall& y)
+{
+    const ConvGeom &g = x.g, &h = y.g;
+    const bool geom = g.N == h.N && g.H == h.H && g.W == h.W && g.C == h.C && g.Ho == h.Ho && g.Wo == h.Wo && g.O == h.O &&
+                      g.kh == h.kh && g.kw == h.kw && g.sh == h.sh && g.sw == h.sw && g.pt == h.pt && g.pl == h.pl;
+    if (!geom || x.kind != y.kind)
+        return false;
+    if (x.kind == 2)
+        return true;
+    return x.b == y.b && x.bias == y.bias && x.act == y.act && x.alpha == y.alpha;
+}
+
+bool writes_in_place(const Step& s)
+{
+    if (s.kind == Step::ADAM || s.kind == Step::ADAM_MULTI)
+        return true;
+    const int t = s.node->type;
+    return t == rt::Node::OP_UPDATE || t == rt::Node::OP_MOMENT_UPDATE || t == rt::Node::OP_MOMENT_UPDATE2 ||
+           t == rt::Node::OP_ADAM_UPDATE;
+}
+
+void outputs_of(const Step& s, std::vector<const dbl_t*>& out)
+{
+    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum})
+        if (n && n->out1)
+            out.push_back(n->out1);
+}
+
+void inputs_of(const Step& s, std::vector<const dbl_t*>& in)
+{
+    std::vector<const dbl_t*> outs;
+    outputs_of(s, outs);
+    auto add = [&](const dbl_t* t) {
+        if (t && std::find(outs.begin(), outs.end(), t) == outs.end() && std::find(in.begin(), in.end(), t) == in.end())
+            in.push_back(t);
+    };
+    add(s.act_ref);
+    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+        if (n)
+        {
+            add(n->in1);
+            add(n->in2);
+            add(n->in3);
+        }
+    for (const Step& g : s.group)
+        inputs_of(g, in);
+}
+
+void pair_convolutions(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
+{
+    std::vector<Step>& st = plan.steps;
+    int n = 0;   // the steps before the first one that writes a variable in place may be re-ordered
+    while (n < (int)st.size() && !writes_in_place(st[n]))
+        ++n;
+    if (n < 2)
+        return;
+    // who produces what, who depends (transitively) on whom, how often a tensor is read
+    std::unordered_map<const dbl_t*, int> producer;
+    std::unordered_map<const dbl_t*, int> reads;
+    std::vector<std::vector<int>> deps(n);
+    std::vector<std::vector<char>> reach(n, std::vector<char>(n, 0));
+    for (int i = 0; i < (int)st.size(); ++i)
+    {
+        std::vector<const dbl_t*> in, out;
+        inputs_of(st[i], in);
+        for (const dbl_t* t : in)
+            ++reads[t];
+        if (i >= n)
+            continue;
+        for (const dbl_t* t : in)
+        {
+            auto f = producer.find(t);
+            if (f == producer.end())
+                continue;
+            deps[i].push_back(f->second);
+            reach[i][f->second] = 1;
+            for (int q = 0; q < n; ++q)
+                if (reach[f->second][q])
+                    reach[i][q] = 1;
+        }
+        outputs_of(st[i], out);
+        for (const dbl_t* t : out)
+            producer[t] = i;
+    }
+    std::vector<ConvCall> call(n);
+    std::vector<char> is_conv(n, 0);
+    for (int i = 0; i < n; ++i)
+        is_conv[i] = conv_call_of(st[i], call[i]) && pairable(call[i]);
+    std::vector<int> partner(n, -1);
+    // forward and input-gradient products with the same filter and epilogue
+    for (int i = 0; i < n; ++i)
+    {
+        if (!is_conv[i] || call[i].kind == 2 || partner[i] >= 0)
+            continue;
+        for (int j = i + 1; j < n; ++j)
+            if (is_conv[j] && partner[j] < 0 && same_call(call[i], call[j]) && !reach[j][i])
+            {
+                partner[i] = j;
+                partner[j] = i;
+                break;
+            }
+    }
+    // filter gradients that only meet in the sum an optimiser step reads
+    std::vector<std::pair<int, int>> dk_pairs;   // (producer of add->in1, producer of add->in2)
+    auto consider = [&](Step& adam) {
+        if (adam.kind != Step::ADAM || !adam.add)
+            return;
+        auto pa = producer.find(adam.add->in1), pb = producer.find(adam.add->in2);
+        if (pa == producer.end() || pb == producer.end() || pa->second == pb->second)
+            return;
+        const int a = pa->second, b = pb->second;
+        if (!is_conv[a] || !is_conv[b] || call[a].kind != 2 || !same_call(call[a], call[b]) || partner[a] >= 0 ||
+            partner[b] >= 0 || call[a].out != adam.add->in1 || call[b].out != adam.add->in2 ||
+            reads[adam.add->in1] != 1 || reads[adam.add->in2] != 1 || keep.count(adam.add->in1) || keep.count(adam.add->in2))
+            return;
+        partner[a] = b;
+        partner[b] = a;
+        dk_pairs.push_back({a, b});
+        adam.grad_sum = adam.add->in1;
+    };
+    for (int i = n; i < (int)st.size(); ++i)
+    {
+        consider(st[i]);
+        for (Step& g : st[i].group)
+            consider(g);
+    }
+    bool any = false;
+    for (int i = 0; i < n; ++i)
+        any = any || partner[i] >= 0;
+    if (!any)
+        return;
+    // merge each pair into one node (named after its first member) and sort again: always the ready
+    // node that stood first in the old order
+    std::vector<int> node_of(n);
+    for (int i = 0; i < n; ++i)
+        node_of[i] = partner[i] >= 0 && partner[i] < i ? partner[i] : i;
+    std::vector<std::vector<int>> succ(n);
+    std::vector<int> waiting(n, 0);
+    for (int i = 0; i < n; ++i)
+        for (int d : deps[i])
+            if (node_of[d] != node_of[i])
+            {
+                succ[node_of[d]].push_back(node_of[i]);
+                ++waiting[node_of[i]];
+            }
+    std::vector<Step> order;
+    std::vector<char> done(n, 0);
+    int nodes = 0, emitted = 0;
+    for (int i = 0; i < n; ++i)
+        nodes += node_of[i] == i;
+    while (emitted < nodes)
+    {
+        int pick = -1;
+        for (int i = 0; i < n && pick < 0; ++i)
+            if (node_of[i] == i && !done[i] && waiting[i] == 0)
+                pick = i;
+        if (pick < 0)
+        {
+            // the merged graph has a cycle: leave the plan as it was
+            for (Step& s : st)
+            {
+                s.grad_sum = nullptr;
+                for (Step& g : s.group)
+                    g.grad_sum = nullptr;
+            }
+            return;
+        }
+        done[pick] = 1;
+        ++emitted;
+        for (int v : succ[pick])
+            --waiting[v];
+        if (partner[pick] < 0)
+            order.push_back(st[pick]);
+        else
+        {
+            int first = pick, second = partner[pick];
+            for (const auto& dk : dk_pairs)   // the contraction is written where the optimiser expects the sum
+                if ((dk.first == first && dk.second == second) || (dk.first == second && dk.second == first))
+                {
+                    first = dk.first;
+                    second = dk.second;
+                }
+            Step pair;
+            pair.kind = Step::CONV_PAIR;
+            pair.node = st[first].node;
+            pair.group = {st[first], st[second]};
+            order.push_back(pair);
+        }
+    }
+    for (int i = n; i < (int)st.size(); ++i)
+        order.push_back(st[i]);
+    st.swap(order);
 }
 
 Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<const dbl_t*>& keep, bool fuse)
@@ -502,10 +760,12 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
         plan.steps.push_back(s);
     }
     gather_adam_steps(plan);
+    if (g_pairing)
+        pair_convolutions(plan, keep);
     if (std::getenv("DCGAN_HIP_PLAN_DUMP"))
     {
         // the launches a run turns into, for inspection
-        static const char* kinds[] = {"node", "conv+epilogue", "act-grad+bias-grad", "adam", "adam-multi"};
+        static const char* kinds[] = {"node", "conv+epilogue", "act-grad+bias-grad", "adam", "adam-multi", "conv pair"};
         std::fprintf(stderr, "plan of %zu nodes -> %zu steps\n", nodes.size(), plan.steps.size());
         for (const Step& s : plan.steps)
             std::fprintf(stderr, "  %-20s %-32s len %zu\n", kinds[s.kind], rt::Node::name_of(s.node->type),
@@ -568,12 +828,29 @@ void issue(const Step& s)
         const float lrt = adam_advance(a);
         if (s.add)
         {
-            dh_adam_item item{a->out1, s.m1->out1, s.m2->out1, s.add->in1, s.add->in2, a->len1, lrt};
+            dh_adam_item item{a->out1, s.m1->out1, s.m2->out1, s.add->in1, s.grad_sum ? nullptr : s.add->in2, a->len1, lrt};
             CK(dh_adam_step_multi(&item, 1, s.m1->cons1, s.m1->cons2, s.m2->cons1, s.m2->cons2, a->cons4, g_stream));
         }
         else
             CK(dh_adam_step(a->out1, s.m1->out1, s.m2->out1, s.m1->in1, s.m1->cons1, s.m1->cons2, s.m2->cons1,
                             s.m2->cons2, lrt, a->cons4, a->len1, g_stream));
+        return;
+    }
+    case Step::CONV_PAIR:
+    {
+        ConvCall a, b;
+        conv_call_of(s.group[0], a);
+        conv_call_of(s.group[1], b);
+        const ConvGeom& g = a.g;
+        if (a.kind == 0)
+            CK(dh_conv2d_fwd_pair(a.a, b.a, a.b, a.out, b.out, g.N, g.H, g.W, g.C, g.kh, g.kw, g.O, g.sh, g.sw, g.pt, g.pl,
+                                  g.Ho, g.Wo, a.bias, a.act, a.alpha, g_stream));
+        else if (a.kind == 1)
+            CK(dh_conv2d_dx_pair(a.a, b.a, a.b, a.out, b.out, g.N, g.Ho, g.Wo, g.O, g.kh, g.kw, g.C, g.sh, g.sw, g.pt, g.pl,
+                                 g.H, g.W, a.bias, a.act, a.alpha, g_stream));
+        else
+            CK(dh_conv2d_dk_pair(a.a, a.b, b.a, b.b, a.out, g.N, g.H, g.W, g.C, g.Ho, g.Wo, g.O, g.kh, g.kw, g.sh, g.sw,
+                                 g.pt, g.pl, g_stream));
         return;
     }
     case Step::ADAM_MULTI:
@@ -584,7 +861,7 @@ void issue(const Step& s)
             rt::Node* a = g.node;
             const float lrt = adam_advance(a);
             items.push_back(dh_adam_item{a->out1, g.m1->out1, g.m2->out1, g.add ? g.add->in1 : g.m1->in1,
-                                         g.add ? g.add->in2 : nullptr, a->len1, lrt});
+                                         g.add && !g.grad_sum ? g.add->in2 : nullptr, a->len1, lrt});
         }
         const Step& f = s.group.front();
         CK(dh_adam_step_multi(items.data(), (int)items.size(), f.m1->cons1, f.m1->cons2, f.m2->cons1, f.m2->cons2,
@@ -664,6 +941,11 @@ void set_fusion(bool on)
     g_fusion = on ? 1 : 0;
 }
 
+void set_pairing(bool on)
+{
+    g_pairing = on;
+}
+
 bool fusion()
 {
     if (g_fusion < 0)
@@ -697,7 +979,10 @@ void run_async(rt::NodesList& tasks)
         it = g_plans.emplace(key, make_plan(tasks.nodes(), g_keep, key.fuse)).first;
     for (const Step& s : it->second.steps)
         issue(s);
+    g_last_launches = (int)it->second.steps.size();
 }
+
+int last_launch_count() { return g_last_launches; }
 
 void run(rt::NodesList& tasks)
 {

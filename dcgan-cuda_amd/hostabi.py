@@ -31,6 +31,7 @@ def load():
         lib.dg_create.argtypes = [C.c_int, C.c_ulonglong]
         lib.dg_destroy.argtypes = [C.c_void_p]
         lib.dg_set_fusion.argtypes = [C.c_int]
+        lib.dg_set_pairing.argtypes = [C.c_int]
         lib.dg_num_vars.argtypes = [C.c_void_p]
         lib.dg_var_size.argtypes = [C.c_void_p, C.c_int]
         lib.dg_var_size.restype = C.c_long
@@ -42,6 +43,7 @@ def load():
         lib.dg_generate.argtypes = [C.c_void_p, _fp]
         lib.dg_eval.argtypes = [C.c_void_p, C.c_char_p, _fp, C.POINTER(C.c_long)]
         lib.dg_last_schedule_size.argtypes = [C.c_void_p]
+        lib.dg_last_launch_count.argtypes = [C.c_void_p]
         for name in ("dg_save_vars", "dg_load_vars", "dg_save_state", "dg_load_state"):
             getattr(lib, name).argtypes = [C.c_void_p, C.c_char_p]
         lib.dg_images_normalize.argtypes = [C.c_char_p, C.c_long, _fp]
@@ -105,6 +107,10 @@ class DcganModel:
     def set_fusion(self, on):
         self.lib.dg_set_fusion(1 if on else 0)
 
+    def set_pairing(self, on):
+        """With fusion: run same-filter convolutions of the two discriminator towers as one launch."""
+        self.lib.dg_set_pairing(1 if on else 0)
+
     def num_vars(self):
         return self.lib.dg_num_vars(self.h)
 
@@ -157,6 +163,10 @@ class DcganModel:
 
     def last_schedule_size(self):
         return self.lib.dg_last_schedule_size(self.h)
+
+    def last_launch_count(self):
+        """Steps (single or fused launches) the last run on the HIP backend issued."""
+        return self.lib.dg_last_launch_count(self.h)
 
     def save_vars(self, path):
         """Trainable variables, creation order; numpy .npz (arr_0, arr_1, ...) when path ends in .npz."""

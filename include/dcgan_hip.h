@@ -26,6 +26,7 @@ extern "C" {
 #endif
 
 #define DH_EINVAL 10001
+#define DH_ENOTSUP 10002 /* a paired launch that this shape cannot take: issue the two single calls instead */
 
 /* Epilogue activations that the convolution entry points can fuse. */
 enum { DH_ACT_NONE = 0, DH_ACT_RELU = 1, DH_ACT_LEAKY = 2, DH_ACT_TANH = 3, DH_ACT_SIGMOID = 4 };
@@ -128,6 +129,28 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx,
 int dh_conv2d_dk(const float* x, const float* dy, float* dk,
                  int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw,
                  int sh, int sw, int pad_top, int pad_left, void* stream);
+
+/* Two instances of the same product in ONE launch: the same filter applied to two sets of
+ * activations of identical shape -- the discriminator on the real and on the generated batch
+ * (dcgan/main.cu:304-307 builds it twice over shared variables).  At batch 64 a single instance
+ * leaves the machine short of workgroups and has to split its contraction; two instances together
+ * need half the splits.
+ *   dh_conv2d_fwd_pair: y1 = conv(x1, k), y2 = conv(x2, k)           (+ the same bias / activation)
+ *   dh_conv2d_dx_pair:  dx1 = dx(dy1, k), dx2 = dx(dy2, k)           (+ the same bias / activation)
+ *   dh_conv2d_dk_pair:  dk = dk(x1, dy1) + dk(x2, dy2), the sum the reference forms with an `add`
+ *                       node when a filter receives gradient along two paths (src/ops/graph.cu:295-308)
+ * They need the 16-byte buffer-load kernel (channel counts divisible by 4, 16-byte aligned tensors
+ * below 2 GiB) and return DH_ENOTSUP otherwise; results agree with the single calls to rounding
+ * (the contraction may be split differently). */
+int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
+                       int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,
+                       const float* bias, int act, float alpha, void* stream);
+int dh_conv2d_dx_pair(const float* dy1, const float* dy2, const float* k, float* dx1, float* dx2, int N, int Ho,
+                      int Wo, int O, int kh, int kw, int C, int sh, int sw, int pad_top, int pad_left, int H, int W,
+                      const float* bias, int act, float alpha, void* stream);
+int dh_conv2d_dk_pair(const float* x1, const float* dy1, const float* x2, const float* dy2, float* dk, int N, int H,
+                      int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left,
+                      void* stream);
 
 /* ---- bias and activations: coalesced, vectorised, one pass over HBM ----------------------------- */
 

@@ -201,6 +201,77 @@ def test_forced_split_counts(be, orc, shape, generic):
         be.lib.dh_debug_force_generic_conv(0)
 
 
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (3, 12, 12, 36, 5, 5, 72, 2),     # partial tiles in m, n and k
+    (2, 32, 32, 64, 5, 5, 128, 2),    # D1 at batch 2
+    (4, 8, 8, 256, 5, 5, 512, 2),     # D3 at batch 4 (split-K)
+    (2, 9, 7, 8, 3, 3, 12, 1),        # stride 1, contraction of one instance not a multiple of 16
+])
+def test_paired_launches(be, orc, shape):
+    """Two instances of a product in one launch (same filter, two sets of activations): forward and
+    input gradient with a fused epilogue give each instance's oracle result; the paired filter
+    gradient gives the sum of the two oracle filter gradients; all repeatable to the bit."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x1, k, dy1 = rand_conv_inputs(31, *shape)
+    x2, _, dy2 = rand_conv_inputs(32, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    bias_c = np.linspace(-0.3, 0.3, C).astype(np.float32)
+    orc.set_threads(8)
+    for rep in range(2):
+        y1, y2 = be.conv2d_pair(x1, x2, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2)
+        g1, g2 = be.conv2d_input_grad_pair(dy1, dy2, k, s, (H, W), bias=bias_c, act=A.ACT_TANH)
+        dk = be.conv2d_kernel_grad_pair(dy1, x1, dy2, x2, s, pads)
+        if rep == 0:
+            first = (y1, y2, g1, g2, dk)
+        else:
+            for a, b in zip(first, (y1, y2, g1, g2, dk)):
+                np.testing.assert_array_equal(a, b)
+    for got, x in ((y1, x1), (y2, x2)):
+        close(got, orc.relu_leaky(orc.bias_add(orc.conv2d(x, k, (s, s)), bias), 0.2), what="paired forward")
+    for got, dy in ((g1, dy1), (g2, dy2)):
+        close(got, orc.tanh(orc.bias_add(orc.conv2d_input_grad(dy, k, s, (H, W)), bias_c)), what="paired input gradient")
+    exp = orc.conv2d_kernel_grad(dy1, x1, s, pads).astype(np.float64) + orc.conv2d_kernel_grad(dy2, x2, s, pads)
+    close(dk, exp.astype(np.float32), scale=max(1.0, float(np.abs(exp).max())), what="paired filter gradient")
+
+
+@pytest.mark.parametrize("shape", [(64, 32, 32, 64, 5, 5, 128, 2), (64, 16, 16, 128, 5, 5, 256, 2), (64, 8, 8, 256, 5, 5, 512, 2)])
+def test_paired_launches_at_batch_64_match_the_single_launches(be, shape):
+    """At the benchmark's shapes (too large for the CPU oracle in a test) the paired launches are
+    compared with the single launches, which the tests above tie to the oracle."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x1, k, dy1 = rand_conv_inputs(41, *shape)
+    x2, _, dy2 = rand_conv_inputs(42, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    y1, y2 = be.conv2d_pair(x1, x2, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2)
+    close(y1, be.conv2d(x1, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), what="forward, first instance")
+    close(y2, be.conv2d(x2, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), what="forward, second instance")
+    g1, g2 = be.conv2d_input_grad_pair(dy1, dy2, k, s, (H, W))
+    close(g1, be.conv2d_input_grad(dy1, k, s, (H, W)), what="input gradient, first instance")
+    close(g2, be.conv2d_input_grad(dy2, k, s, (H, W)), what="input gradient, second instance")
+    dk = be.conv2d_kernel_grad_pair(dy1, x1, dy2, x2, s, pads)
+    exp = be.conv2d_kernel_grad(dy1, x1, s, pads).astype(np.float64) + be.conv2d_kernel_grad(dy2, x2, s, pads)
+    close(dk, exp.astype(np.float32), scale=max(1.0, float(np.abs(exp).max())), what="filter gradient")
+
+
+def test_paired_launch_refuses_what_it_cannot_take(be):
+    """Channel counts that are not multiples of 4 have no paired kernel: DH_ENOTSUP, not a wrong result."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    x, k, dy = rand_conv_inputs(1, 2, 8, 8, 3, 5, 5, 6, 2)
+    with pytest.raises(A.HipError, match="10002"):
+        be.conv2d_pair(x, x, k, (2, 2))
+    with pytest.raises(A.HipError, match="10002"):
+        be.conv2d_kernel_grad_pair(dy, x, dy, x, 2, (3, 3))
+
+
 def test_dk_is_reproducible(be):
     """Split-K partial sums are reduced in a fixed order: two runs give identical bits."""
     x, k, dy = rand_conv_inputs(3, 8, 16, 16, 128, 5, 5, 256, 2)

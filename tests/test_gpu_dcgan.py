@@ -27,11 +27,14 @@ def cpu_dump(tmp_path_factory):
 
 
 def gpu_dump(fusion):
+    """fusion: False (one launch per instruction), True (fused launches, the two discriminator towers'
+    convolutions paired), "unpaired" (fused launches, every convolution on its own)."""
     import __graft_entry__ as ge
     pkg = ge.load_package()
     model = pkg.hostabi.DcganModel(BATCH, SEED, "GPU")
     try:
-        model.set_fusion(fusion)
+        model.set_fusion(bool(fusion))
+        model.set_pairing(fusion != "unpaired")
         w, z, x = dr.synthetic(BATCH, SEED, pkg.hostabi.var_shapes())
         for name, val in w.items():
             model.set_var(name, val)
@@ -39,10 +42,35 @@ def gpu_dump(fusion):
         return dr.collect(model), model.last_schedule_size()
     finally:
         model.set_fusion(False)
+        model.set_pairing(True)
         model.close()
 
 
-@pytest.mark.parametrize("fusion", [False, True])
+def test_paired_plan_is_shorter():
+    """With pairing the discriminator step issues nine launches fewer: layers 1-3 forward, input
+    gradient and filter gradient of the two towers each become one launch."""
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    counts = {}
+    for pairing in (True, False):
+        model = pkg.hostabi.DcganModel(BATCH, SEED, "GPU")
+        try:
+            model.set_fusion(True)
+            model.set_pairing(pairing)
+            w, z, x = dr.synthetic(BATCH, SEED, pkg.hostabi.var_shapes())
+            for name, val in w.items():
+                model.set_var(name, val)
+            model.set_inputs(z, x)
+            model.d_step()
+            counts[pairing] = model.last_launch_count()
+        finally:
+            model.set_fusion(False)
+            model.set_pairing(True)
+            model.close()
+    assert counts[False] - counts[True] == 9, counts
+
+
+@pytest.mark.parametrize("fusion", [False, True, "unpaired"])
 def test_dcgan_layers_losses_gradients_and_one_adam_iteration(cpu_dump, fusion):
     print("fusion", fusion, flush=True)
     got, _ = gpu_dump(fusion)
