@@ -41,12 +41,13 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; averages over the launches of
 # one kernel symbol), each scaled by the same counter's reading for the calibration copy.  The
 # summaries are kept under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000)
-    "conv_igemm_fast<fwd,128x128>": 78.5e6,
-    "conv_igemm_fast<dx,128x128>": 78.0e6,
-    "conv_igemm_fast<dk,128x128>": 116.1e6,
-    "conv_igemm_fast<dx,128x64>": 34.4e6,
-    "conv_igemm<fwd,128x64,sv>": 21.7e6,
+MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
+    # launch-weighted over the single and the paired instantiation of a tag
+    "conv_igemm_fast<fwd,128x128>": 91.9e6,     # 6 single launches of 78.2 MB, 3 paired of 119.1 MB per iteration
+    "conv_igemm_fast<dx,128x128>": 79.1e6,      # 6 x 77.9 MB, 2 x 82.4 MB
+    "conv_igemm_fast<dk,128x128>": 157.8e6,     # 3 x 116.2 MB, 3 x 199.5 MB
+    "conv_igemm_fast<dx,128x64>": 66.1e6,       # 3 x 34.9 MB, 1 x 159.8 MB
+    "fwd_thin": 21.7e6,
     "conv_igemm<dk,128x64,sv>": 25.6e6,
     "dx_few_channels": 27.2e6,
 }
