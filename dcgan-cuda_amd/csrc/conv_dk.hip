@@ -25,10 +25,17 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
     if (pair && !takes_fast_path(veca, vecb))
         return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const long slabs_one = (p.phase[0].K + BK - 1) / BK;
-    p.pair_slabs = pair ? (int)slabs_one : 0;
     const TileCfg cfg = pick_tile(p.phase[0].M, O);
-    const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn);
-    p.splitk = pick_splitk(wgs, slabs_one * (pair ? 2 : 1));
+    if (takes_fast_path(veca, vecb))
+    {
+        p.skip = N % BK == 0;
+        plan_split<MODE_DK>(p, p.phase, 1, cfg, pair);
+    }
+    else
+    {
+        const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn);
+        p.splitk = pick_splitk(wgs, slabs_one * (pair ? 2 : 1));
+    }
     if (p.splitk > 1)
     {
         void* ws;

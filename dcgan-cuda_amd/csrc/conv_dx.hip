@@ -75,7 +75,13 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     const TileCfg cfg = pick_tile(max_m, C);
     for (int q = 0; q < n_live; ++q)
         total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;
-    p.splitk = pick_splitk(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances, min_slabs);
+    if (takes_fast_path(veca, vecb))
+    {
+        p.skip = O % BK == 0;
+        plan_split<MODE_DX>(p, all, n_live, cfg, pair);
+    }
+    else
+        p.splitk = pick_splitk(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances, min_slabs);
     if (p.splitk > 1)
     {
         void* ws;

@@ -202,6 +202,54 @@ def test_forced_split_counts(be, orc, shape, generic):
 
 
 @pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (16, 8, 8, 16, 5, 5, 32, 2),     # one image slab per pixel; tiles span several pixels
+    (32, 4, 4, 32, 5, 5, 16, 2),     # 2x2 outputs: every tap is padding for some pixel
+    (16, 9, 7, 16, 5, 5, 16, 2),     # odd extents: one-sided padding differs between the axes
+    (48, 5, 5, 16, 5, 5, 32, 2),     # 48 images: pixel boundaries fall inside row tiles
+    (16, 6, 6, 16, 3, 3, 16, 1),     # stride 1: a single phase, taps skipped at all four borders
+    (16, 7, 7, 16, 4, 4, 16, 3),     # stride 3, even filter
+    (128, 4, 4, 16, 5, 5, 16, 2),    # one pixel per 128-row tile: the box of live taps is exact
+    (16, 2, 2, 16, 5, 5, 16, 2),     # a single output pixel
+    (16, 1, 1, 16, 5, 5, 16, 2),     # 1x1 image: one live tap
+    (256, 4, 4, 16, 5, 5, 16, 2),    # two row tiles per pixel
+])
+@pytest.mark.parametrize("splits", [0, 5])
+def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
+    """Shapes on which the buffer-load kernel leaves out the k-slabs whose taps fall into the
+    padding (channel and image counts divisible by 16): forward, input gradient and filter gradient,
+    single and paired, automatic split and a forced one, against the oracle."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, "splits", splits, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(31, *shape)
+    x2, _, dy2 = rand_conv_inputs(32, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    orc.set_threads(8)
+    exp_f = orc.relu_leaky(orc.bias_add(orc.conv2d(x, k, (s, s)), bias), 0.2)
+    exp_x = orc.conv2d_input_grad(dy, k, s, (H, W))
+    exp_k = orc.conv2d_kernel_grad(dy, x, s, pads)
+    be.lib.dh_debug_force_splitk(splits)
+    try:
+        close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), exp_f, what="fwd")
+        close(be.conv2d_input_grad(dy, k, s, (H, W)), exp_x, what="dx")
+        kscale = max(1.0, float(np.abs(exp_k).max()))
+        close(be.conv2d_kernel_grad(dy, x, s, pads), exp_k, scale=kscale, what="dk")
+        if N <= 64:
+            exp_f2 = orc.relu_leaky(orc.bias_add(orc.conv2d(x2, k, (s, s)), bias), 0.2)
+            got1, got2 = be.conv2d_pair(x, x2, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2)
+            close(got1, exp_f, what="fwd pair 1"), close(got2, exp_f2, what="fwd pair 2")
+            got1, got2 = be.conv2d_input_grad_pair(dy, dy2, k, s, (H, W))
+            close(got1, exp_x, what="dx pair 1")
+            close(got2, orc.conv2d_input_grad(dy2, k, s, (H, W)), what="dx pair 2")
+            exp_k2 = exp_k + orc.conv2d_kernel_grad(dy2, x2, s, pads)
+            close(be.conv2d_kernel_grad_pair(dy, x, dy2, x2, s, pads), exp_k2, scale=2 * kscale, what="dk pair")
+    finally:
+        be.lib.dh_debug_force_splitk(0)
+
+
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
     (3, 12, 12, 36, 5, 5, 72, 2),     # partial tiles in m, n and k
     (2, 32, 32, 64, 5, 5, 128, 2),    # D1 at batch 2
     (4, 8, 8, 256, 5, 5, 512, 2),     # D3 at batch 4 (split-K)

@@ -147,3 +147,59 @@ def test_adam_many_variables_in_one_launch(be, orc):
     got = be.adam_step_multi(items, 0.5, 0.999, 1e-8)
     for (gp, gm, gv), (ep, em, ev) in zip(got, expect):
         close(gm, em), close(gv, ev), close(gp, ep)
+
+
+def test_empty_inputs(be):
+    """Zero-length tensors: the element-wise, bias, dense and Adam entry points return success and
+    write nothing; the losses and argmax, whose result divides by the element count, refuse them;
+    a null tensor with a non-zero length is refused everywhere."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    lib = be.lib
+    guard = np.arange(8, dtype=np.float32) + 1
+    buf, src = A.Buf.from_numpy(guard), A.Buf.from_numpy(guard)
+    ok = lambda rc: A.check(rc)
+    for fn in (lib.dh_relu, lib.dh_tanh, lib.dh_sigmoid):
+        ok(fn(src.ptr, buf.ptr, 0, None))
+    ok(lib.dh_relu_leaky(src.ptr, buf.ptr, 0, 0.2, None))
+    for fn in (lib.dh_relu_grad, lib.dh_tanh_grad, lib.dh_sigmoid_grad, lib.dh_add, lib.dh_mse_grad,
+               lib.dh_sigmoid_cross_entropy_grad):
+        ok(fn(src.ptr, src.ptr, buf.ptr, 0, None))
+    ok(lib.dh_leaky_relu_grad(src.ptr, src.ptr, buf.ptr, 0.2, 0, None))
+    ok(lib.dh_bias_add(src.ptr, src.ptr, buf.ptr, 0, 8, None))
+    ok(lib.dh_bias_add(src.ptr, src.ptr, buf.ptr, 8, 0, None))
+    ok(lib.dh_bias_grad(src.ptr, buf.ptr, 8, 0, None))
+    ok(lib.dh_mat_sum_rows(src.ptr, buf.ptr, 0, 8, None))
+    ok(lib.dh_gemm_nn(src.ptr, src.ptr, None, buf.ptr, 0, 4, 2, None))
+    ok(lib.dh_gemm_tn(src.ptr, src.ptr, buf.ptr, 2, 4, 0, None))
+    ok(lib.dh_moment_update(buf.ptr, src.ptr, 0.5, 0.5, 0, None))
+    ok(lib.dh_moment_update2(buf.ptr, src.ptr, 0.5, 0.5, 0, None))
+    ok(lib.dh_adam_update(buf.ptr, src.ptr, src.ptr, 0.1, 1e-8, 0, None))
+    ok(lib.dh_adam_step(buf.ptr, buf.ptr, buf.ptr, src.ptr, 0.5, 0.5, 0.9, 0.1, 0.1, 1e-8, 0, None))
+    ok(lib.dh_adam_step_multi(None, 0, 0.5, 0.5, 0.9, 0.1, 1e-8, None))
+    item = (A.AdamItem * 1)()
+    item[0].p = item[0].m = item[0].v = buf.ptr
+    item[0].g1, item[0].g2, item[0].n, item[0].lrt = src.ptr, None, 0, 0.1
+    ok(lib.dh_adam_step_multi(item, 1, 0.5, 0.5, 0.9, 0.1, 1e-8, None))
+    ok(lib.dh_memset0(buf.ptr, 0, None))
+    ok(lib.dh_stream_sync(None))
+    np.testing.assert_array_equal(buf.numpy(), guard)
+    # the column sum of a matrix without rows is the zero vector; a product over an empty inner
+    # extent is the bias (or zero)
+    ok(lib.dh_bias_grad(src.ptr, buf.ptr, 0, 8, None))
+    np.testing.assert_array_equal(buf.numpy(), np.zeros(8, np.float32))
+    buf.write(guard)
+    ok(lib.dh_gemm_nn(src.ptr, src.ptr, src.ptr, buf.ptr, 2, 0, 4, None))
+    np.testing.assert_array_equal(buf.numpy(), np.concatenate([guard[:4], guard[:4]]))
+    ok(lib.dh_gemm_nn(src.ptr, src.ptr, None, buf.ptr, 2, 0, 4, None))
+    np.testing.assert_array_equal(buf.numpy(), np.zeros(8, np.float32))
+    for bad in (lambda: lib.dh_sigmoid_cross_entropy(src.ptr, src.ptr, buf.ptr, 0, None),
+                lambda: lib.dh_mse(src.ptr, src.ptr, buf.ptr, 0, 4, None),
+                lambda: lib.dh_argmax_acc(src.ptr, src.ptr, buf.ptr, 4, 0, None),
+                lambda: lib.dh_relu(None, buf.ptr, 8, None),
+                lambda: lib.dh_add(src.ptr, None, buf.ptr, 8, None),
+                lambda: lib.dh_bias_add(src.ptr, None, buf.ptr, 2, 4, None),
+                lambda: lib.dh_gemm_nn(src.ptr, None, None, buf.ptr, 2, 2, 2, None),
+                lambda: lib.dh_adam_step(buf.ptr, buf.ptr, None, src.ptr, 0.5, 0.5, 0.9, 0.1, 0.1, 1e-8, 8, None)):
+        with pytest.raises(A.HipError):
+            A.check(bad())
