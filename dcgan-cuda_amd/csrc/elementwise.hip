@@ -38,8 +38,33 @@ struct OpSigmoidGrad { __device__ float operator()(float s, float d) const { ret
 struct OpAdd { __device__ float operator()(float a, float b) const { return a + b; } };
 struct OpSceGrad { float inv_n; __device__ float operator()(float y, float x) const { return (1.f / (1.f + expf(-x)) - y) * inv_n; } };
 struct OpMseGrad { float coeff; __device__ float operator()(float y, float yh) const { return coeff * (yh - y); } };
-struct OpMoment { float a, b; __device__ float operator()(float m, float g) const { return a * m + b * g; } };
-struct OpMoment2 { float a, b; __device__ float operator()(float v, float g) const { return a * v + b * g * g; } };
+// The optimiser's arithmetic with contraction into fused multiply-adds switched off: every product
+// and sum is rounded on its own, as in the reference's CPU kernels (src/cpu/ops.hxx moment_update /
+// adam_update compiled without FMA).  Left to itself the compiler fuses a*m + b*g into one FMA, and
+// not the same one at every place the expression is inlined, so the separate kernels, the
+// single-pass step and the multi-variable step would differ in the last bit.
+__device__ __forceinline__ float moment1(float a, float m, float b, float g)
+{
+#pragma clang fp contract(off)
+    const float am = a * m, bg = b * g;
+    return am + bg;
+}
+__device__ __forceinline__ float moment2(float a, float v, float b, float g)
+{
+#pragma clang fp contract(off)
+    const float av = a * v, bg = b * g;
+    const float bgg = bg * g;
+    return av + bgg;
+}
+__device__ __forceinline__ float adam_apply1(float p, float m, float v, float lrt, float eps)
+{
+#pragma clang fp contract(off)
+    const float num = lrt * m, den = sqrtf(v) + eps;
+    const float q = num / den;
+    return p - q;
+}
+struct OpMoment { float a, b; __device__ float operator()(float m, float g) const { return moment1(a, m, b, g); } };
+struct OpMoment2 { float a, b; __device__ float operator()(float v, float g) const { return moment2(a, v, b, g); } };
 
 template <class F>
 __global__ __launch_bounds__(TPB) void map1(const float* __restrict__ x, float* __restrict__ out, size_t n, bool vec, F f)
@@ -264,8 +289,31 @@ __global__ __launch_bounds__(TPB) void colsum_stage2(const float* __restrict__ p
     if (lane == 0) out[c] = s;
 }
 
-int run_colsum(const char* who, const float* a, const float* act_ref, float* dz, float* db, size_t rows,
-               size_t cols, ActGrad g, bool fused, void* stream)
+// How run_colsum cuts the rows: `chunks` ranges of rows_per_chunk rows (G rows side by side for
+// narrow matrices), col_tiles tiles of 256 columns.
+struct ColsumCut { uint32_t G; unsigned col_tiles; size_t chunks, rows_per_chunk; };
+
+ColsumCut colsum_cut(size_t rows, size_t cols)
+{
+    ColsumCut c;
+    c.G = cols <= TPB ? (uint32_t)(TPB / cols) : 0;
+    c.col_tiles = cols <= TPB ? 1u : (unsigned)((cols + TPB - 1) / TPB);
+    // aim at ~4 workgroups per compute unit, at least 8 row groups each
+    size_t row_groups = c.G ? (rows + c.G - 1) / c.G : rows;
+    size_t chunks = ((size_t)num_cus() * 4 + c.col_tiles - 1) / c.col_tiles;
+    if (chunks > (row_groups + 7) / 8) chunks = (row_groups + 7) / 8;
+    if (chunks < 1) chunks = 1;
+    if (chunks > 65535) chunks = 65535;
+    size_t rows_per_chunk = (rows + chunks - 1) / chunks;
+    if (c.G) rows_per_chunk = (rows_per_chunk + c.G - 1) / c.G * c.G;
+    c.rows_per_chunk = rows_per_chunk;
+    c.chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
+    return c;
+}
+
+// db: the column sums (both stages).  parts_out: the per-range sums of stage 1 only, left to the caller.
+int run_colsum(const char* who, const float* a, const float* act_ref, float* dz, float* db, float* parts_out,
+               size_t rows, size_t cols, ActGrad g, bool fused, void* stream)
 {
     DH_TRY(ensure_init());
     if (cols == 0) return 0;
@@ -274,45 +322,36 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     hipStream_t st = as_stream(stream);
     if (rows == 0)
     {
-        if (db)
+        float* zero = parts_out ? parts_out : db;   // no rows: one range, whose sums are zero
+        if (zero)
         {
-            hipLaunchKernelGGL(fill_zero, dim3(grid_for(cols)), dim3(TPB), 0, st, db, cols, false);
+            hipLaunchKernelGGL(fill_zero, dim3(grid_for(cols)), dim3(TPB), 0, st, zero, cols, false);
             DH_LAUNCH_CHECK(who);
         }
         return 0;
     }
-    const uint32_t G = cols <= TPB ? (uint32_t)(TPB / cols) : 0;
-    const unsigned col_tiles = cols <= TPB ? 1u : (unsigned)((cols + TPB - 1) / TPB);
-    // aim at ~4 workgroups per compute unit, at least 8 row groups each
-    size_t row_groups = G ? (rows + G - 1) / G : rows;
-    size_t chunks = ((size_t)num_cus() * 4 + col_tiles - 1) / col_tiles;
-    if (chunks > (row_groups + 7) / 8) chunks = (row_groups + 7) / 8;
-    if (chunks < 1) chunks = 1;
-    if (chunks > 65535) chunks = 65535;
-    size_t rows_per_chunk = (rows + chunks - 1) / chunks;
-    if (G) rows_per_chunk = (rows_per_chunk + G - 1) / G * G;
-    chunks = (rows + rows_per_chunk - 1) / rows_per_chunk;
-    float* partial = nullptr;
-    if (db)
+    const ColsumCut cut = colsum_cut(rows, cols);
+    float* partial = parts_out;
+    if (db && !partial)
     {
         void* ws;
-        DH_TRY(workspace(chunks * cols * sizeof(float), &ws, st));
+        DH_TRY(workspace(cut.chunks * cols * sizeof(float), &ws, st));
         partial = static_cast<float*>(ws);
     }
-    dim3 grid(col_tiles, (unsigned)chunks);
+    dim3 grid(cut.col_tiles, (unsigned)cut.chunks);
     ProfScope prof(fused ? "hbm:activation gradient + column sums (12 B/elem)" : "hbm:column sums (4 B/elem)",
                    (fused ? 12.0 : 4.0) * rows * cols, st);
     if (fused)
         hipLaunchKernelGGL(colsum_stage1<true>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
-                           (uint32_t)cols, G, rows_per_chunk, g);
+                           (uint32_t)cols, cut.G, cut.rows_per_chunk, g);
     else
         hipLaunchKernelGGL(colsum_stage1<false>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
-                           (uint32_t)cols, G, rows_per_chunk, g);
+                           (uint32_t)cols, cut.G, cut.rows_per_chunk, g);
     DH_LAUNCH_CHECK(who);
-    if (db)
+    if (db && !parts_out)
     {
         hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + TPB / 64 - 1) / (TPB / 64))), dim3(TPB), 0, st,
-                           partial, db, (uint32_t)cols, (uint32_t)chunks);
+                           partial, db, (uint32_t)cols, (uint32_t)cut.chunks);
         DH_LAUNCH_CHECK(who);
     }
     return 0;
@@ -406,24 +445,24 @@ __global__ __launch_bounds__(TPB) void adam_update_kernel(float* __restrict__ p,
             float4 pp = reinterpret_cast<float4*>(p)[i];
             const float4 mm = reinterpret_cast<const float4*>(m)[i];
             const float4 vv = reinterpret_cast<const float4*>(v)[i];
-            pp.x = pp.x - lrt * mm.x / (sqrtf(vv.x) + eps);
-            pp.y = pp.y - lrt * mm.y / (sqrtf(vv.y) + eps);
-            pp.z = pp.z - lrt * mm.z / (sqrtf(vv.z) + eps);
-            pp.w = pp.w - lrt * mm.w / (sqrtf(vv.w) + eps);
+            pp.x = adam_apply1(pp.x, mm.x, vv.x, lrt, eps);
+            pp.y = adam_apply1(pp.y, mm.y, vv.y, lrt, eps);
+            pp.z = adam_apply1(pp.z, mm.z, vv.z, lrt, eps);
+            pp.w = adam_apply1(pp.w, mm.w, vv.w, lrt, eps);
             reinterpret_cast<float4*>(p)[i] = pp;
         }
         done = n4 * 4;
     }
     for (size_t i = done + tid; i < n; i += stride)
-        p[i] = p[i] - lrt * m[i] / (sqrtf(v[i]) + eps);
+        p[i] = adam_apply1(p[i], m[i], v[i], lrt, eps);
 }
 
 __device__ __forceinline__ void adam1(float& p, float& m, float& v, float g, float b1, float c1, float b2, float c2,
                                       float lrt, float eps)
 {
-    m = b1 * m + c1 * g;
-    v = b2 * v + c2 * g * g;
-    p = p - lrt * m / (sqrtf(v) + eps);
+    m = moment1(b1, m, c1, g);
+    v = moment2(b2, v, c2, g);
+    p = adam_apply1(p, m, v, lrt, eps);
 }
 
 __global__ __launch_bounds__(TPB) void adam_step_kernel(float* __restrict__ p, float* __restrict__ m, float* __restrict__ v,
@@ -472,8 +511,24 @@ struct AdamBatch
     float lrt[ADAM_MAX_ITEMS];
     unsigned first_block[ADAM_MAX_ITEMS + 1];
     unsigned char vec[ADAM_MAX_ITEMS];  // every pointer of the item 16-byte aligned
+    // > 1: the gradient is the sum of that many vectors of n elements (row-range sums of a bias
+    // gradient); such an item gives each of its elements to one wavefront
+    unsigned parts1[ADAM_MAX_ITEMS], parts2[ADAM_MAX_ITEMS];
     int count;
 };
+
+// Sum of `parts` vectors at element e, one wavefront: lane l adds parts l, l + 64, ... in that order,
+// the lane sums are combined by the shuffle tree of colsum_stage2 -- the same additions in the same
+// order as the bias gradient's second stage, whose place this takes.  Valid in lane 0.
+__device__ __forceinline__ float sum_of_parts(const float* __restrict__ g, unsigned parts, size_t n, size_t e, unsigned lane)
+{
+    float s = 0.f;
+    for (unsigned q = lane; q < parts; q += 64)
+        s += g[(size_t)q * n + e];
+    for (int off = 32; off > 0; off >>= 1)
+        s += __shfl_down(s, off, 64);
+    return s;
+}
 
 __global__ __launch_bounds__(TPB) void adam_step_multi_kernel(const AdamBatch batch, float b1, float c1, float b2, float c2,
                                                               float eps)
@@ -488,6 +543,19 @@ __global__ __launch_bounds__(TPB) void adam_step_multi_kernel(const AdamBatch ba
     const float* __restrict__ g2 = batch.g2[item];
     const size_t n = batch.n[item];
     const float lrt = batch.lrt[item];
+    if (batch.parts1[item] > 1 || batch.parts2[item] > 1)
+    {
+        const size_t e = (size_t)(blockIdx.x - batch.first_block[item]) * (TPB / 64) + (threadIdx.x >> 6);
+        const unsigned lane = threadIdx.x & 63;
+        if (e >= n)
+            return;
+        float ga = batch.parts1[item] > 1 ? sum_of_parts(g1, batch.parts1[item], n, e, lane) : g1[e];
+        if (g2)
+            ga += batch.parts2[item] > 1 ? sum_of_parts(g2, batch.parts2[item], n, e, lane) : g2[e];
+        if (lane == 0)
+            adam1(p[e], m[e], v[e], ga, b1, c1, b2, c2, lrt, eps);
+        return;
+    }
     const size_t base = (size_t)(blockIdx.x - batch.first_block[item]) * ADAM_BLOCK;
     if (batch.vec[item])
     {
@@ -575,13 +643,34 @@ int dh_bias_add(const float* z, const float* b, float* out, size_t rows, size_t 
 int dh_bias_grad(const float* dz, float* db, size_t rows, size_t cols, void* stream)
 {
     if (!db && cols) return fail(DH_EINVAL, "dh_bias_grad: null result");
-    return run_colsum("dh_bias_grad", dz, nullptr, nullptr, db, rows, cols, ActGrad{DH_ACT_NONE, 0.f}, false, stream);
+    return run_colsum("dh_bias_grad", dz, nullptr, nullptr, db, nullptr, rows, cols, ActGrad{DH_ACT_NONE, 0.f}, false, stream);
+}
+
+size_t dh_bias_grad_part_count(size_t rows, size_t cols)
+{
+    if (rows == 0 || cols == 0 || ensure_init() != 0) return rows == 0 && cols != 0 ? 1 : 0;
+    return colsum_cut(rows, cols).chunks;
+}
+
+int dh_bias_grad_parts(const float* dz, float* parts, size_t rows, size_t cols, void* stream)
+{
+    if (!parts && cols) return fail(DH_EINVAL, "dh_bias_grad_parts: null result");
+    return run_colsum("dh_bias_grad_parts", dz, nullptr, nullptr, nullptr, parts, rows, cols, ActGrad{DH_ACT_NONE, 0.f}, false,
+                      stream);
 }
 
 int dh_act_bias_grad(const float* act_ref, const float* dout, float* dz, float* db, size_t rows, size_t cols,
                      int act, float alpha, void* stream)
 {
-    return run_colsum("dh_act_bias_grad", dout, act_ref, dz, db, rows, cols, ActGrad{act, alpha}, true, stream);
+    return run_colsum("dh_act_bias_grad", dout, act_ref, dz, db, nullptr, rows, cols, ActGrad{act, alpha}, true, stream);
+}
+
+int dh_act_bias_grad_parts(const float* act_ref, const float* dout, float* dz, float* parts, size_t rows, size_t cols,
+                           int act, float alpha, void* stream)
+{
+    if (!parts && cols) return fail(DH_EINVAL, "dh_act_bias_grad_parts: null result");
+    return run_colsum("dh_act_bias_grad_parts", dout, act_ref, dz, nullptr, parts, rows, cols, ActGrad{act, alpha}, true,
+                      stream);
 }
 
 int dh_mat_sum_rows(const float* a, float* out, size_t rows, size_t cols, void* stream)
@@ -693,16 +782,20 @@ int dh_adam_step_multi(const dh_adam_item* items, int count, float m_decay, floa
             if (it.n == 0)
                 continue;
             if (!it.p || !it.m || !it.v || !it.g1) return fail(DH_EINVAL, "dh_adam_step_multi: null tensor in item %d", at);
-            const size_t nb = (it.n + ADAM_BLOCK - 1) / ADAM_BLOCK;
+            const bool in_parts = it.g1_parts > 1 || (it.g2 && it.g2_parts > 1);
+            if (it.g1_parts > 0xffffffffu || it.g2_parts > 0xffffffffu)
+                return fail(DH_EINVAL, "dh_adam_step_multi: too many gradient parts in item %d", at);
+            const size_t nb = in_parts ? (it.n + TPB / 64 - 1) / (TPB / 64) : (it.n + ADAM_BLOCK - 1) / ADAM_BLOCK;
             if (nb > 0x7fffffffu - blocks) return fail(DH_EINVAL, "dh_adam_step_multi: too many elements");
             const int i = batch.count++;
             batch.p[i] = it.p; batch.m[i] = it.m; batch.v[i] = it.v; batch.g1[i] = it.g1; batch.g2[i] = it.g2;
             batch.n[i] = it.n; batch.lrt[i] = it.lrt;
+            batch.parts1[i] = (unsigned)it.g1_parts; batch.parts2[i] = it.g2 ? (unsigned)it.g2_parts : 0;
             batch.vec[i] = aligned16(it.p) && aligned16(it.m) && aligned16(it.v) && aligned16(it.g1) &&
                            (!it.g2 || aligned16(it.g2));
             batch.first_block[i] = blocks;
             blocks += (unsigned)nb;
-            bytes += (it.g2 ? 32.0 : 28.0) * it.n;
+            bytes += (24.0 + 4.0 * (it.g1_parts > 1 ? it.g1_parts : 1) + (it.g2 ? 4.0 * (it.g2_parts > 1 ? it.g2_parts : 1) : 0.0)) * it.n;
         }
         if (batch.count == 0)
             continue;

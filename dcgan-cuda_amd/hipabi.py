@@ -52,6 +52,7 @@ _SIGS = {
     "dh_conv2d_dk_pair": [_vp] * 5 + [_i] * 13 + [_vp],
     "dh_bias_add": [_vp, _vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad": [_vp, _vp, _sz, _sz, _vp],
+    "dh_bias_grad_parts": [_vp, _vp, _sz, _sz, _vp],
     "dh_mat_sum_rows": [_vp, _vp, _sz, _sz, _vp],
     "dh_relu": [_vp, _vp, _sz, _vp],
     "dh_relu_leaky": [_vp, _vp, _sz, _f, _vp],
@@ -63,6 +64,7 @@ _SIGS = {
     "dh_sigmoid_grad": [_vp, _vp, _vp, _sz, _vp],
     "dh_add": [_vp, _vp, _vp, _sz, _vp],
     "dh_act_bias_grad": [_vp, _vp, _vp, _vp, _sz, _sz, _i, _f, _vp],
+    "dh_act_bias_grad_parts": [_vp, _vp, _vp, _vp, _sz, _sz, _i, _f, _vp],
     "dh_sigmoid_cross_entropy": [_vp, _vp, _vp, _sz, _vp],
     "dh_sigmoid_cross_entropy_grad": [_vp, _vp, _vp, _sz, _vp],
     "dh_mse": [_vp, _vp, _vp, _sz, _sz, _vp],
@@ -78,7 +80,9 @@ _SIGS = {
     "dh_adam_step_multi": [_vp, _i, _f, _f, _f, _f, _f, _vp],
     "dh_sgd_update": [_vp, _vp, _vp, _sz, _vp],
 }
-_RESTYPES = {"dh_version": C.c_char_p, "dh_last_error": C.c_char_p, "dh_workspace_bytes": _sz}
+# name -> result type, or (result type, argtypes)
+_RESTYPES = {"dh_version": C.c_char_p, "dh_last_error": C.c_char_p, "dh_workspace_bytes": _sz,
+             "dh_bias_grad_part_count": (_sz, [_sz, _sz])}
 
 _lib = None
 
@@ -97,8 +101,7 @@ def load():
             fn.restype = _i
         for name, res in _RESTYPES.items():
             fn = getattr(lib, name)
-            fn.argtypes = []
-            fn.restype = res
+            fn.restype, fn.argtypes = res if isinstance(res, tuple) else (res, [])
         _lib = lib
     return _lib
 
@@ -172,7 +175,7 @@ def device_info():
 class AdamItem(C.Structure):
     """dh_adam_item of include/dcgan_hip.h."""
     _fields_ = [("p", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("g1", C.c_void_p), ("g2", C.c_void_p),
-                ("n", C.c_size_t), ("lrt", C.c_float)]
+                ("n", C.c_size_t), ("lrt", C.c_float), ("g1_parts", C.c_size_t), ("g2_parts", C.c_size_t)]
 
 
 class Timer:
@@ -364,6 +367,24 @@ class HipBackend:
                                         self.stream))
         return dz.numpy(), db.numpy()
 
+    def bias_grad_parts(self, dz):
+        """Row-range sums [parts, cols] whose sum over axis 0 (in dh_bias_grad's order) is the bias gradient."""
+        d, = self._up(dz)
+        cols = dz.shape[-1]
+        parts = self.lib.dh_bias_grad_part_count(dz.size // cols, cols)
+        out = Buf((parts, cols))
+        check(self.lib.dh_bias_grad_parts(d.ptr, out.ptr, dz.size // cols, cols, self.stream))
+        return out.numpy()
+
+    def act_bias_grad_parts(self, act_ref, dout, act, alpha=0.0):
+        r, d = self._up(act_ref, dout)
+        cols = dout.shape[-1]
+        parts = self.lib.dh_bias_grad_part_count(dout.size // cols, cols)
+        dz, out = Buf(dout.shape), Buf((parts, cols))
+        check(self.lib.dh_act_bias_grad_parts(r.ptr, d.ptr, dz.ptr, out.ptr, dout.size // cols, cols, act, alpha,
+                                              self.stream))
+        return dz.numpy(), out.numpy()
+
     def mat_sum_rows(self, a):
         d, = self._up(a)
         out = Buf((a.shape[0],))
@@ -495,14 +516,16 @@ class HipBackend:
         return dp.numpy(), dm.numpy(), dv.numpy()
 
     def adam_step_multi(self, items, beta1, beta2, eps):
-        """items: [(p, m, v, g1, g2 or None, lrt)] -> [(p, m, v)] after one step, all in one launch."""
+        """items: [(p, m, v, g1, g2 or None, lrt)] -> [(p, m, v)] after one step, all in one launch.
+        A gradient with one more axis than p is taken as row-range sums [parts, n] (see bias_grad_parts)."""
         arr = (AdamItem * len(items))()
         bufs = []
         for i, (p, m, v, g1, g2, lrt) in enumerate(items):
             dp, dm, dv, dg = self._up(p, m, v, g1)
             dh = Buf.from_numpy(g2) if g2 is not None else None
             bufs.append((dp, dm, dv, dg, dh))
-            arr[i] = AdamItem(dp.ptr, dm.ptr, dv.ptr, dg.ptr, dh.ptr if dh else None, dp.size, lrt)
+            parts = [g.shape[0] if g is not None and g.ndim == p.ndim + 1 else 0 for g in (g1, g2)]
+            arr[i] = AdamItem(dp.ptr, dm.ptr, dv.ptr, dg.ptr, dh.ptr if dh else None, dp.size, lrt, parts[0], parts[1])
         one = np.float32(1)
         check(self.lib.dh_adam_step_multi(arr, len(items), beta1, one - np.float32(beta1), beta2,
                                           one - np.float32(beta2), eps, self.stream))

@@ -214,6 +214,12 @@ struct Step
     const dbl_t* act_ref = nullptr;  // ACT_BIAS_GRAD: tensor the activation gradient reads
     std::vector<Step> group;     // ADAM_MULTI: the ADAM steps issued as one launch; CONV_PAIR: the two convolution steps
     const dbl_t* grad_sum = nullptr;  // ADAM: gradient tensor that already holds the sum of both contributions
+    // A bias gradient read by nothing but the optimiser is left as its row-range sums and added up
+    // inside the optimiser launch (defer_bias_sums).  Producer (ACT_BIAS_GRAD, or NODE mat_sum_cols):
+    // where the sums go.  ADAM: for each of its two gradient slots, the sums and their count.
+    dbl_t* parts = nullptr;
+    const dbl_t* g_parts[2] = {nullptr, nullptr};
+    std::size_t g_nparts[2] = {0, 0};
 };
 
 int act_code(const rt::Node* n)
@@ -322,6 +328,92 @@ void gather_adam_steps(Plan& plan)
         moved.swap(rest);
     }
     plan.steps.swap(kept);
+}
+
+// ---- bias gradients summed inside the optimiser launch ---------------------------------------------
+// A bias gradient is a column sum in two kernels: sums over ranges of rows, then the sum of those.
+// When nothing but optimiser steps of one launch reads it, the second kernel is dropped: the producer
+// writes its row-range sums to a buffer of its own and dh_adam_step_multi adds them, in the same
+// order, while it reads the gradient (15 launches of a DCGAN iteration, each of them pure latency).
+std::unordered_map<const dbl_t*, std::pair<dbl_t*, std::size_t>> g_parts_pool;   // bias gradient -> (buffer, floats)
+
+dbl_t* parts_buffer(const dbl_t* grad, std::size_t floats)
+{
+    auto& slot = g_parts_pool[grad];
+    if (slot.second < floats)
+    {
+        if (slot.first)
+            CK(dh_free(slot.first));
+        void* q = nullptr;
+        CK(dh_malloc(&q, floats * sizeof(dbl_t)));
+        slot = {static_cast<dbl_t*>(q), floats};
+    }
+    return slot.first;
+}
+
+void defer_bias_sums(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
+{
+    // the optimiser steps of the plan, by address
+    std::vector<Step*> adams;
+    for (Step& s : plan.steps)
+    {
+        if (s.kind == Step::ADAM)
+            adams.push_back(&s);
+        for (Step& g : s.group)
+            if (s.kind == Step::ADAM_MULTI)
+                adams.push_back(&g);
+    }
+    for (Step& s : plan.steps)
+    {
+        rt::Node* sum = s.kind == Step::ACT_BIAS_GRAD ? s.sum
+                        : s.kind == Step::NODE && s.node->type == rt::Node::OP_MAT_SUM_COLS ? s.node : nullptr;
+        if (!sum || keep.count(sum->out1))
+            continue;
+        const dbl_t* db = sum->out1;
+        // every reader must be a gradient slot of an optimiser step
+        bool ok = true;
+        std::vector<std::pair<Step*, int>> slots;
+        for (Step& other : plan.steps)
+        {
+            if (&other == &s || other.kind == Step::ADAM || other.kind == Step::ADAM_MULTI)
+                continue;
+            std::unordered_set<const dbl_t*> touched;
+            tensors_of(other, touched);
+            for (const Step& g : other.group)
+                tensors_of(g, touched);
+            if (touched.count(db))
+                ok = false;
+        }
+        for (Step* a : adams)
+        {
+            const dbl_t* g1 = a->add ? a->add->in1 : a->m1->in1;
+            const dbl_t* g2 = a->add && !a->grad_sum ? a->add->in2 : nullptr;
+            if (g1 == db) slots.push_back({a, 0});
+            if (g2 == db) slots.push_back({a, 1});
+            // anything else of that step touching the tensor (its variable, a moment) rules it out
+            for (const dbl_t* t : {(const dbl_t*)a->node->out1, (const dbl_t*)a->m1->out1, (const dbl_t*)a->m2->out1})
+                if (t == db)
+                    ok = false;
+        }
+        if (!ok || slots.empty())
+            continue;
+        // a stand-alone step without an `add` goes through dh_adam_step, which takes plain gradients
+        for (auto& sl : slots)
+            for (Step& top : plan.steps)
+                if (&top == sl.first && top.kind == Step::ADAM && !top.add)
+                    ok = false;
+        if (!ok)
+            continue;
+        const std::size_t nparts = dh_bias_grad_part_count(sum->len1, sum->len2);
+        if (nparts < 2)
+            continue;
+        s.parts = parts_buffer(db, nparts * sum->len2);
+        for (auto& sl : slots)
+        {
+            sl.first->g_parts[sl.second] = s.parts;
+            sl.first->g_nparts[sl.second] = nparts;
+        }
+    }
 }
 
 // ---- paired convolutions ---------------------------------------------------------------------------
@@ -762,6 +854,7 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
     gather_adam_steps(plan);
     if (g_pairing)
         pair_convolutions(plan, keep);
+    defer_bias_sums(plan, keep);
     if (std::getenv("DCGAN_HIP_PLAN_DUMP"))
     {
         // the launches a run turns into, for inspection
@@ -772,6 +865,24 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
                          (std::size_t)s.node->len1);
     }
     return plan;
+}
+
+// The optimiser step of one variable as dh_adam_step_multi takes it: gradient g1 (+ g2 when the
+// reference formed it with an `add` node that is not already folded into a paired filter gradient),
+// either of them possibly as row-range sums (defer_bias_sums).
+dh_adam_item adam_item(const Step& s, float lrt)
+{
+    rt::Node* a = s.node;
+    const dbl_t* g1 = s.add ? s.add->in1 : s.m1->in1;
+    const dbl_t* g2 = s.add && !s.grad_sum ? s.add->in2 : nullptr;
+    dh_adam_item item{};
+    item.p = a->out1; item.m = s.m1->out1; item.v = s.m2->out1;
+    item.g1 = s.g_parts[0] ? s.g_parts[0] : g1;
+    item.g2 = g2 ? (s.g_parts[1] ? s.g_parts[1] : g2) : nullptr;
+    item.n = a->len1; item.lrt = lrt;
+    item.g1_parts = s.g_parts[0] ? s.g_nparts[0] : 0;
+    item.g2_parts = g2 && s.g_parts[1] ? s.g_nparts[1] : 0;
+    return item;
 }
 
 void issue(const Step& s)
@@ -788,6 +899,12 @@ void issue(const Step& s)
                 CK(dh_relu_grad(s.act_ref, n->in2, n->out1, n->len1, g_stream));
             else
                 CK(dh_leaky_relu_grad(s.act_ref, n->in2, n->out1, n->cons1, n->len1, g_stream));
+            return;
+        }
+        if (s.parts)
+        {
+            // bias gradient left as row-range sums for the optimiser launch
+            CK(dh_bias_grad_parts(n->in1, s.parts, n->len1, n->len2, g_stream));
             return;
         }
         kernel_f f = n->type >= 0 && n->type < 512 ? kernels_list[n->type] : nullptr;
@@ -818,8 +935,12 @@ void issue(const Step& s)
         rt::Node* g = s.node;
         const int act = g->type == rt::Node::OP_RELU_GRAD ? DH_ACT_RELU
                         : g->type == rt::Node::OP_LEAKY_RELU_GRAD ? DH_ACT_LEAKY : DH_ACT_TANH;
-        CK(dh_act_bias_grad(s.act_ref, g->in2, g->out1, s.sum->out1, s.sum->len1, s.sum->len2, act, g->cons1,
-                            g_stream));
+        if (s.parts)
+            CK(dh_act_bias_grad_parts(s.act_ref, g->in2, g->out1, s.parts, s.sum->len1, s.sum->len2, act, g->cons1,
+                                      g_stream));
+        else
+            CK(dh_act_bias_grad(s.act_ref, g->in2, g->out1, s.sum->out1, s.sum->len1, s.sum->len2, act, g->cons1,
+                                g_stream));
         return;
     }
     case Step::ADAM:
@@ -828,7 +949,7 @@ void issue(const Step& s)
         const float lrt = adam_advance(a);
         if (s.add)
         {
-            dh_adam_item item{a->out1, s.m1->out1, s.m2->out1, s.add->in1, s.grad_sum ? nullptr : s.add->in2, a->len1, lrt};
+            const dh_adam_item item = adam_item(s, lrt);
             CK(dh_adam_step_multi(&item, 1, s.m1->cons1, s.m1->cons2, s.m2->cons1, s.m2->cons2, a->cons4, g_stream));
         }
         else
@@ -860,8 +981,7 @@ void issue(const Step& s)
         {
             rt::Node* a = g.node;
             const float lrt = adam_advance(a);
-            items.push_back(dh_adam_item{a->out1, g.m1->out1, g.m2->out1, g.add ? g.add->in1 : g.m1->in1,
-                                         g.add && !g.grad_sum ? g.add->in2 : nullptr, a->len1, lrt});
+            items.push_back(adam_item(g, lrt));
         }
         const Step& f = s.group.front();
         CK(dh_adam_step_multi(items.data(), (int)items.size(), f.m1->cons1, f.m1->cons2, f.m2->cons1, f.m2->cons2,

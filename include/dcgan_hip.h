@@ -160,6 +160,13 @@ int dh_bias_add(const float* z, const float* b, float* out, size_t rows, size_t 
 /* db[c] = sum_r dz[r,c].  conv2d_bias_add_grad lowers to this
  * (src/ops/conv2d-bias-add-grad.cu:29-31); replaces gpu::mat_sum_cols (src/gpu/sum.cu:112-151). */
 int dh_bias_grad(const float* dz, float* db, size_t rows, size_t cols, void* stream);
+/* The first half of dh_bias_grad only: parts[q*cols + c] = sum of column c over the q-th range of rows,
+ * for the dh_bias_grad_part_count(rows, cols) ranges the matrix is cut into (`parts` must hold that
+ * many times cols floats).  The sum over q, in the order dh_bias_grad uses, is left to the consumer:
+ * dh_adam_step_multi takes a gradient in this form (no counterpart in the reference, whose
+ * mat_sum_cols is one kernel per column block, src/gpu/sum.cu:112-151). */
+size_t dh_bias_grad_part_count(size_t rows, size_t cols);
+int dh_bias_grad_parts(const float* dz, float* parts, size_t rows, size_t cols, void* stream);
 /* out[r] = sum_c a[r,c].  Replaces gpu::mat_sum_rows (src/gpu/sum.cu:69-108). */
 int dh_mat_sum_rows(const float* a, float* out, size_t rows, size_t cols, void* stream);
 /* Replace vect_relu / vect_relu_leaky (src/gpu/relu.cu:26-55), vect_sigmoid / vect_tanh
@@ -184,6 +191,9 @@ int dh_add(const float* a, const float* b, float* out, size_t n, void* stream);
  * Fuses leaky_relu_grad + mat_sum_cols of the reference's backward node list. */
 int dh_act_bias_grad(const float* act_ref, const float* dout, float* dz, float* db,
                      size_t rows, size_t cols, int act, float alpha, void* stream);
+/* The same with the column sums left as row-range sums (see dh_bias_grad_parts). */
+int dh_act_bias_grad_parts(const float* act_ref, const float* dout, float* dz, float* parts,
+                           size_t rows, size_t cols, int act, float alpha, void* stream);
 
 /* ---- losses --------------------------------------------------------------------------------------- */
 
@@ -231,7 +241,11 @@ int dh_adam_step(float* p, float* m, float* v, const float* g, float m_decay, fl
  * most of them bias vectors of a few hundred elements).  Item i uses the gradient g1, or g1 + g2
  * when g2 is not null: that sum is what the reference forms with a separate `add` node when a
  * variable receives gradient along two paths (src/ops/graph.cu:295-308, src/cpu/ops.hxx:933-938).
- * lrt is per item because every variable keeps its own step counter (src/ops/adam-update.cu:45). */
+ * lrt is per item because every variable keeps its own step counter (src/ops/adam-update.cu:45).
+ * A gradient may also be handed over as the row-range sums dh_bias_grad_parts / dh_act_bias_grad_parts
+ * leave behind: g1_parts > 1 says that g1 holds g1_parts vectors of n elements whose sum is the gradient
+ * (likewise g2_parts).  They are added here exactly as dh_bias_grad would have added them, so the
+ * result is the same to the bit and the bias gradient's second kernel is never launched. */
 typedef struct dh_adam_item
 {
     float* p;
@@ -241,6 +255,8 @@ typedef struct dh_adam_item
     const float* g2;
     size_t n;
     float lrt;
+    size_t g1_parts; /* 0 or 1: g1 is the gradient itself */
+    size_t g2_parts;
 } dh_adam_item;
 int dh_adam_step_multi(const dh_adam_item* items, int count, float m_decay, float m_gain, float v_decay,
                        float v_gain, float eps, void* stream);

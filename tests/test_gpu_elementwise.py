@@ -203,3 +203,34 @@ def test_empty_inputs(be):
                 lambda: lib.dh_adam_step(buf.ptr, buf.ptr, None, src.ptr, 0.5, 0.5, 0.9, 0.1, 0.1, 1e-8, 8, None)):
         with pytest.raises(A.HipError):
             A.check(bad())
+
+
+@pytest.mark.parametrize("rows,cols", [(4096, 64), (65536, 3), (1024, 512), (16384, 128), (7, 5), (64, 8192)])
+def test_bias_gradient_in_parts_through_adam(be, orc, rows, cols):
+    """dh_bias_grad_parts / dh_act_bias_grad_parts leave the column sums as row-range sums;
+    dh_adam_step_multi fed with them gives, to the bit, what it gives when fed with dh_bias_grad's
+    result -- with one gradient, with two, and with one of the two in plain form."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    rng = np.random.default_rng(rows + cols)
+    z = rng.uniform(-2, 2, (rows, cols)).astype(np.float32)
+    d1 = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    d2 = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
+    parts1 = be.bias_grad_parts(d1)
+    assert parts1.shape == (be.lib.dh_bias_grad_part_count(rows, cols), cols)
+    plain1 = be.bias_grad(d1)
+    close(parts1.astype(np.float64).sum(axis=0).astype(np.float32), orc.bias_grad(d1), scale=max(1.0, np.sqrt(rows)))
+    dz_ref, plain2 = be.act_bias_grad(z, d2, A.ACT_LEAKY, 0.2)
+    dz, parts2 = be.act_bias_grad_parts(z, d2, A.ACT_LEAKY, 0.2)
+    np.testing.assert_array_equal(dz, dz_ref)
+    p = rng.standard_normal(cols).astype(np.float32)
+    m = (rng.standard_normal(cols) * 0.1).astype(np.float32)
+    v = (rng.uniform(0, 1, cols) * 0.01).astype(np.float32)
+    lrt = 1e-3
+    want = be.adam_step_multi([(p, m, v, plain1, None, lrt), (p, m, v, plain1, plain2, lrt), (p, m, v, plain2, plain1, lrt)],
+                              0.5, 0.999, 1e-8)
+    got = be.adam_step_multi([(p, m, v, parts1, None, lrt), (p, m, v, parts1, parts2, lrt), (p, m, v, plain2, parts1, lrt)],
+                             0.5, 0.999, 1e-8)
+    for w, g in zip(want, got):
+        for a, b in zip(w, g):
+            np.testing.assert_array_equal(a, b)
