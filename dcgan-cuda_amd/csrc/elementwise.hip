@@ -273,6 +273,90 @@ __global__ __launch_bounds__(TPB) void colsum_stage1(const float* __restrict__ a
     }
 }
 
+// Stage 1 for column counts divisible by 4: a lane owns 4 adjacent columns (one 16-byte access per
+// tensor and row; ALIGNED says whether the tensors allow it, otherwise the same 4 elements are
+// accessed one by one), G4 = 256 / (cols / 4) rows lie side by side for matrices of up to 1024
+// columns, wider ones are cut into tiles of 1024 columns.  Same two-level order of additions as the
+// scalar kernel: a lane adds its rows serially, lanes of the same columns are added in lane order.
+template <bool FUSED, bool ALIGNED>
+__global__ __launch_bounds__(TPB) void colsum_stage1_v4(const float* __restrict__ a, const float* __restrict__ act_ref,
+                                                        float* __restrict__ dz, float* __restrict__ partial,
+                                                        size_t rows, uint32_t cols, uint32_t G4, size_t rows_per_chunk,
+                                                        ActGrad g)
+{
+    __shared__ float4 lds[TPB];
+    const uint32_t t = threadIdx.x;
+    const uint32_t c4n = cols / 4;
+    const size_t r_begin = (size_t)blockIdx.y * rows_per_chunk;
+    size_t r_end = r_begin + rows_per_chunk;
+    if (r_end > rows) r_end = rows;
+    uint32_t rsub = 0, col4, step = 1;
+    bool live;
+    if (G4 >= 1)
+    {
+        rsub = t / c4n;
+        col4 = t - rsub * c4n;
+        live = t < G4 * c4n;
+        step = G4;
+    }
+    else
+    {
+        col4 = blockIdx.x * TPB + t;
+        live = col4 < c4n;
+    }
+    auto load4 = [](const float* q) {
+        if (ALIGNED)
+            return *reinterpret_cast<const float4*>(q);
+        return make_float4(q[0], q[1], q[2], q[3]);
+    };
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live)
+    {
+#pragma unroll 4
+        for (size_t r = r_begin + rsub; r < r_end; r += step)
+        {
+            const size_t idx = r * cols + (size_t)col4 * 4;
+            float4 v = load4(a + idx);
+            if (FUSED)
+            {
+                const float4 ref = load4(act_ref + idx);
+                v.x = g(ref.x, v.x); v.y = g(ref.y, v.y); v.z = g(ref.z, v.z); v.w = g(ref.w, v.w);
+                if (ALIGNED)
+                    *reinterpret_cast<float4*>(dz + idx) = v;
+                else
+                {
+                    dz[idx] = v.x; dz[idx + 1] = v.y; dz[idx + 2] = v.z; dz[idx + 3] = v.w;
+                }
+            }
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+    }
+    if (G4 >= 1)
+    {
+        lds[t] = acc;
+        __syncthreads();
+        if (t < c4n)
+        {
+            float4 s = lds[t];
+            for (uint32_t q = 1; q < G4; ++q)
+            {
+                const float4 o = lds[q * c4n + t];
+                s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+            }
+            if (partial)
+            {
+                float* dst = partial + (size_t)blockIdx.y * cols + (size_t)t * 4;
+                dst[0] = s.x; dst[1] = s.y; dst[2] = s.z; dst[3] = s.w;
+            }
+        }
+    }
+    else if (live && partial)
+    {
+        float* dst = partial + (size_t)blockIdx.y * cols + (size_t)col4 * 4;
+        dst[0] = acc.x; dst[1] = acc.y; dst[2] = acc.z; dst[3] = acc.w;
+    }
+}
+
 // One wavefront per column: lane l adds the per-range sums l, l+64, ... in that order, then the 64
 // lane sums are combined by a fixed shuffle tree.
 __global__ __launch_bounds__(TPB) void colsum_stage2(const float* __restrict__ partial, float* __restrict__ out,
@@ -290,18 +374,20 @@ __global__ __launch_bounds__(TPB) void colsum_stage2(const float* __restrict__ p
 }
 
 // How run_colsum cuts the rows: `chunks` ranges of rows_per_chunk rows (G rows side by side for
-// narrow matrices), col_tiles tiles of 256 columns.
-struct ColsumCut { uint32_t G; unsigned col_tiles; size_t chunks, rows_per_chunk; };
+// narrow matrices), col_tiles tiles of 256 lanes; with vec4 a lane holds 4 adjacent columns.
+struct ColsumCut { bool vec4; uint32_t G; unsigned col_tiles; size_t chunks, rows_per_chunk; };
 
 ColsumCut colsum_cut(size_t rows, size_t cols)
 {
     ColsumCut c;
-    c.G = cols <= TPB ? (uint32_t)(TPB / cols) : 0;
-    c.col_tiles = cols <= TPB ? 1u : (unsigned)((cols + TPB - 1) / TPB);
-    // aim at ~4 workgroups per compute unit, at least 8 row groups each
+    c.vec4 = cols % 4 == 0;
+    const size_t lanes = c.vec4 ? cols / 4 : cols;   // lanes that one row occupies
+    c.G = lanes <= TPB ? (uint32_t)(TPB / lanes) : 0;
+    c.col_tiles = lanes <= TPB ? 1u : (unsigned)((lanes + TPB - 1) / TPB);
+    // aim at ~4 workgroups per compute unit, at least 4 row groups each
     size_t row_groups = c.G ? (rows + c.G - 1) / c.G : rows;
     size_t chunks = ((size_t)num_cus() * 4 + c.col_tiles - 1) / c.col_tiles;
-    if (chunks > (row_groups + 7) / 8) chunks = (row_groups + 7) / 8;
+    if (chunks > (row_groups + 3) / 4) chunks = (row_groups + 3) / 4;
     if (chunks < 1) chunks = 1;
     if (chunks > 65535) chunks = 65535;
     size_t rows_per_chunk = (rows + chunks - 1) / chunks;
@@ -341,12 +427,16 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     dim3 grid(cut.col_tiles, (unsigned)cut.chunks);
     ProfScope prof(fused ? "hbm:activation gradient + column sums (12 B/elem)" : "hbm:column sums (4 B/elem)",
                    (fused ? 12.0 : 4.0) * rows * cols, st);
-    if (fused)
-        hipLaunchKernelGGL(colsum_stage1<true>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
-                           (uint32_t)cols, cut.G, cut.rows_per_chunk, g);
-    else
-        hipLaunchKernelGGL(colsum_stage1<false>, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows,
-                           (uint32_t)cols, cut.G, cut.rows_per_chunk, g);
+    const bool al = aligned16(a) && (!fused || (aligned16(act_ref) && aligned16(dz)));
+#define DH_COLSUM_LAUNCH(KERNEL) \
+    hipLaunchKernelGGL(KERNEL, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows, (uint32_t)cols, cut.G, cut.rows_per_chunk, g)
+    if (cut.vec4 && fused && al) DH_COLSUM_LAUNCH((colsum_stage1_v4<true, true>));
+    else if (cut.vec4 && fused) DH_COLSUM_LAUNCH((colsum_stage1_v4<true, false>));
+    else if (cut.vec4 && al) DH_COLSUM_LAUNCH((colsum_stage1_v4<false, true>));
+    else if (cut.vec4) DH_COLSUM_LAUNCH((colsum_stage1_v4<false, false>));
+    else if (fused) DH_COLSUM_LAUNCH(colsum_stage1<true>);
+    else DH_COLSUM_LAUNCH(colsum_stage1<false>);
+#undef DH_COLSUM_LAUNCH
     DH_LAUNCH_CHECK(who);
     if (db && !parts_out)
     {

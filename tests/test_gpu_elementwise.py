@@ -234,3 +234,23 @@ def test_bias_gradient_in_parts_through_adam(be, orc, rows, cols):
     for w, g in zip(want, got):
         for a, b in zip(w, g):
             np.testing.assert_array_equal(a, b)
+
+
+def test_column_sums_of_unaligned_tensors(be, orc):
+    """Column counts divisible by 4 take the kernel whose lanes own 4 adjacent columns; tensors that
+    do not start on a 16-byte boundary go through its element-wise accesses."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    rng = np.random.default_rng(9)
+    rows, cols = 777, 36
+    z = rng.uniform(-2, 2, rows * cols + 1).astype(np.float32)
+    d = rng.uniform(-1, 1, rows * cols + 1).astype(np.float32)
+    dz_buf, db = A.Buf(rows * cols + 1), A.Buf(cols)
+    zb, dbuf = A.Buf.from_numpy(z), A.Buf.from_numpy(d)
+    A.check(be.lib.dh_act_bias_grad(zb.ptr + 4, dbuf.ptr + 4, dz_buf.ptr + 4, db.ptr, rows, cols, A.ACT_LEAKY, 0.2, None))
+    z2, d2 = z[1:].reshape(rows, cols), d[1:].reshape(rows, cols)
+    exp = orc.leaky_relu_grad(z2, d2, 0.2)
+    np.testing.assert_array_equal(dz_buf.numpy()[1:].reshape(rows, cols), exp)
+    close(db.numpy(), orc.bias_grad(exp), scale=np.sqrt(rows))
+    A.check(be.lib.dh_bias_grad(dbuf.ptr + 4, db.ptr, rows, cols, None))
+    close(db.numpy(), orc.bias_grad(d2), scale=np.sqrt(rows))
