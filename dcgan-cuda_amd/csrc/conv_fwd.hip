@@ -34,16 +34,14 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
         return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const TileCfg cfg = pick_tile(p.phase[0].M, O);
     const int instances = pair ? 2 : 1;
+    const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
     if (takes_fast_path(veca, vecb))
     {
-        p.skip = C % BK == 0;
+        p.skip = C % BK == 0 && skipping_pays(wgs);
         plan_split<MODE_FWD>(p, p.phase, 1, cfg, pair);
     }
     else
-    {
-        const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
         p.splitk = pick_splitk(wgs, (p.phase[0].K + BK - 1) / BK);
-    }
     if (p.splitk > 1)
     {
         void* ws;
