@@ -43,10 +43,10 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # summaries are kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
     # launch-weighted over the single and the paired instantiation of a tag
-    "conv_igemm_fast<fwd,128x128>": 91.9e6,     # 6 single launches of 78.2 MB, 3 paired of 119.1 MB per iteration
-    "conv_igemm_fast<dx,128x128>": 79.1e6,      # 6 x 77.9 MB, 2 x 82.4 MB
-    "conv_igemm_fast<dk,128x128>": 157.8e6,     # 3 x 116.2 MB, 3 x 199.5 MB
-    "conv_igemm_fast<dx,128x64>": 66.1e6,       # 3 x 34.9 MB, 1 x 159.8 MB
+    "conv_igemm_fast<fwd,128x128>": 112.5e6,    # 6 single launches of 84.6 MB, 3 paired of 168.2 MB per iteration
+    "conv_igemm_fast<dx,128x128>": 98.3e6,      # 6 x 93.8 MB, 2 x 111.9 MB
+    "conv_igemm_fast<dk,128x128>": 191.4e6,     # 3 x 126.1 MB, 3 x 256.7 MB
+    "conv_igemm_fast<dx,128x64>": 41.5e6,       # 3 x 34.4 MB, 1 x 62.7 MB
     "fwd_thin": 21.7e6,
     "conv_igemm<dk,128x64,sv>": 25.6e6,
     "dx_few_channels": 27.2e6,

@@ -77,7 +77,7 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
         total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;
     if (takes_fast_path(veca, vecb))
     {
-        p.skip = O % BK == 0 && skipping_pays(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances);
+        p.skip = p.posmajor = O % BK == 0 && skipping_pays(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances);
         plan_split<MODE_DX>(p, all, n_live, cfg, pair);
     }
     else

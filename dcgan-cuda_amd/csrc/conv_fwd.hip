@@ -37,7 +37,7 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
     if (takes_fast_path(veca, vecb))
     {
-        p.skip = C % BK == 0 && skipping_pays(wgs);
+        p.skip = p.posmajor = C % BK == 0 && skipping_pays(wgs);
         plan_split<MODE_FWD>(p, p.phase, 1, cfg, pair);
     }
     else
