@@ -48,7 +48,7 @@ MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FET
     "conv_igemm_fast<dk,128x128>": 191.4e6,     # 3 x 126.1 MB, 3 x 256.7 MB
     "conv_igemm_fast<dx,128x64>": 41.5e6,       # 3 x 34.4 MB, 1 x 62.7 MB
     "fwd_thin": 21.7e6,
-    "conv_igemm<dk,128x64,sv>": 25.6e6,
+    "dk_thin": 25.5e6,
     "dx_few_channels": 27.2e6,
 }
 

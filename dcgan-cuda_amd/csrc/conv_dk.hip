@@ -11,6 +11,27 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
     DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     const bool pair = x2 != nullptr || dy2 != nullptr;
     if (!x || !dy || !dk || (pair && (!x2 || !dy2))) return fail(DH_EINVAL, "%s: null tensor", who);
+    if (!pair && !g_force_generic && aligned16(dk))
+    {
+        float* part = nullptr;
+        int splits = 0;
+        const int rc = conv_dk_thin(x, dy, &part, &splits, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left,
+                                    as_stream(stream));
+        if (rc == 0)
+        {
+            // the slices are added in slice order, 16 lanes per output
+            const size_t n = (size_t)kh * kw * C * O;
+            size_t blocks = (n / 4 * 16 + 255) / 256;
+            if (blocks > 4096) blocks = 4096;
+            ProfScope prof("hbm:splitk_reduce (4 B x (splits + 1) per output)", 4.0 * n * (splits + 1), as_stream(stream));
+            hipLaunchKernelGGL(splitk_reduce_wide, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), part, dk,
+                               (float*)nullptr, (const float*)nullptr, n, n, O, splits, (int)DH_ACT_NONE, 0.f);
+            DH_LAUNCH_CHECK("splitk_reduce_wide launch");
+            return 0;
+        }
+        if (rc != 1)
+            return rc;
+    }
     ConvParams p{};
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = x; p.b_src = dy; p.out = dk; p.bias = nullptr; p.act = DH_ACT_NONE; p.alpha = 0.f;

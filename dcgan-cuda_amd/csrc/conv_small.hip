@@ -289,6 +289,209 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
     }
 }
 
+
+// ---- filter gradient of a thin input ------------------------------------------------------------
+// dk[(di,dj,c), o] = sum over pixels of x[b, i*sh+di-pt, j*sw+dj-pl, c] * dy[b,i,j,o] for a filter
+// with at most 96 elements per output channel and at most 64 output channels (the discriminator's
+// first layer: 75 x 64).  As an implicit GEMM it is a 75-row product whose "im2col" operand has to
+// be gathered element by element (3 channels); here a wavefront takes segments of 16 neighbouring
+// output pixels of one image row and stages, per segment, the kh input rows they touch and their
+// 16 dy pixels in LDS.  Element ((di, dj, c), j) of the gathered operand is then
+//     patch[di][(dj*C + c) + j*sw*C]
+// -- a strided view of the staged rows, read straight into the MFMA registers with no gather at all.
+// The four wavefronts of a workgroup work on different segments and add their accumulators through
+// LDS in wavefront order; each workgroup writes one slice of partial sums, which the caller adds
+// up (fixed order, so the result is repeatable to the bit).
+typedef float dt_f32x16 __attribute__((ext_vector_type(16)));
+constexpr int DT_SEG = 16;                    // output pixels per segment
+constexpr int DT_XMAX = 640;                  // floats of one staged input patch (kh rows)
+constexpr int DT_OMAX = 64;                   // output channels, and the LDS stride of a dy pixel
+constexpr int DT_XPL = DT_XMAX / 64;          // patch elements a lane loads
+constexpr int DT_WAVE_LDS = DT_XMAX + DT_SEG * DT_OMAX + 64;   // floats per wavefront (the last 64: zeros)
+constexpr int DT_MT = 3, DT_NT = 2;           // 32x32 MFMA tiles of the result
+static_assert(4 * DT_WAVE_LDS >= DT_MT * 32 * DT_OMAX, "the accumulators of a workgroup are added in its staging memory");
+
+struct ThinDkParams
+{
+    const float* x;
+    const float* dy;
+    float* part;          // [workgroup][M][O]
+    int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
+    int M;                // kh * kw * C
+    int row;              // kw * C
+    int rsw;              // floats of a staged input row: (DT_SEG - 1) * sw * C + kw * C
+    int rs;               // its LDS stride (bank-conflict-free fragment reads)
+    int segs_per_row, total_segs, segs_per_wave;
+    FastDiv fd_segs_per_row, fd_Ho, fd_rsw, fd_row, fd_O4;
+};
+
+__global__ __launch_bounds__(256) void dk_thin(const ThinDkParams p)
+{
+    __shared__ __attribute__((aligned(16))) float lds[4 * DT_WAVE_LDS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float* lx = lds + wave * DT_WAVE_LDS;
+    float* ld = lx + DT_XMAX;
+    float* lzero = ld + DT_SEG * DT_OMAX;
+    lzero[lane] = 0.f;
+    const int s_begin = ((int)blockIdx.x * 4 + wave) * p.segs_per_wave;
+    const int s_end = min(p.total_segs, s_begin + p.segs_per_wave);
+
+    // patch elements of this lane: e = lane + 64 q -> (row r, column col) of the staged rows
+    // (row and column packed into one register: r << 16 | col; r = 0x7fff for a lane without element)
+    int x_rc[DT_XPL];
+#pragma unroll
+    for (int q = 0; q < DT_XPL; ++q)
+    {
+        const int e = lane + 64 * q;
+        uint32_t r, col;
+        p.fd_rsw.divmod(e, r, col);
+        x_rc[q] = (int)(((int)r < p.kh ? r : 0x7fffu) << 16 | col);
+    }
+    // dy elements of this lane: 16-byte pieces f = lane + 64 q -> (pixel, channel quad)
+    int d_pix[4], d_o4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+    {
+        uint32_t pix, o4;
+        p.fd_O4.divmod(lane + 64 * q, pix, o4);
+        d_pix[q] = (int)pix < DT_SEG ? (int)pix : (1 << 28);
+        d_o4[q] = (int)o4;
+    }
+    // MFMA fragments: A[m = (di, dj*C + c)][k = pixel], B[k = pixel][n = o]; lanes 32-63 hold the second pixel
+    const int l32 = lane & 31, half = lane >> 5;
+    // (rows and columns past the result's extents read a zero word, with a step of zero)
+    int a_ptr[DT_MT], b_ptr[DT_NT];   // offsets into this wavefront's LDS
+    int a_step[DT_MT], b_step[DT_NT];
+    const int zero_at = DT_XMAX + DT_SEG * DT_OMAX + lane;
+#pragma unroll
+    for (int mt = 0; mt < DT_MT; ++mt)
+    {
+        const int m = mt * 32 + l32;
+        uint32_t di, mp;
+        p.fd_row.divmod(m, di, mp);
+        a_ptr[mt] = m < p.M ? (int)di * p.rs + (int)mp + half * p.sw * p.C : zero_at;
+        a_step[mt] = m < p.M ? p.sw * p.C : 0;
+    }
+#pragma unroll
+    for (int nt = 0; nt < DT_NT; ++nt)
+    {
+        const int n = nt * 32 + l32;
+        b_ptr[nt] = n < p.O ? DT_XMAX + half * DT_OMAX + n : zero_at;
+        b_step[nt] = n < p.O ? DT_OMAX : 0;
+    }
+    dt_f32x16 acc[DT_MT][DT_NT];
+#pragma unroll
+    for (int mt = 0; mt < DT_MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < DT_NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[mt][nt][r] = 0.f;
+
+    float xv[DT_XPL];
+    float4 dv[4];
+    auto load = [&](int s) {
+        uint32_t bi, js, b, i;
+        p.fd_segs_per_row.divmod(s, bi, js);
+        p.fd_Ho.divmod(bi, b, i);
+        const int j0 = (int)js * DT_SEG;
+        const int ih0 = (int)i * p.sh - p.pt;
+        const int g0 = (j0 * p.sw - p.pl) * p.C;      // first staged column, in floats from the row start
+        const float* xrow = p.x + ((size_t)b * p.H) * p.W * p.C;
+        const ptrdiff_t base = (ptrdiff_t)ih0 * p.W * p.C + g0;
+        // every lane loads (from the start of the image where its element does not exist) and the value
+        // is dropped afterwards, so that the loads are issued back to back
+#pragma unroll
+        for (int q = 0; q < DT_XPL; ++q)
+        {
+            const int r = x_rc[q] >> 16, col = x_rc[q] & 0xffff;
+            const int ih = ih0 + r, g = g0 + col;
+            const bool ok = (unsigned)ih < (unsigned)p.H && (unsigned)g < (unsigned)(p.W * p.C);
+            const float v = xrow[ok ? base + r * p.W * p.C + col : 0];
+            xv[q] = ok ? v : 0.f;
+        }
+        const float* drow = p.dy + (((size_t)b * p.Ho + i) * p.Wo + j0) * p.O;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const bool ok = d_pix[q] < DT_SEG && j0 + d_pix[q] < p.Wo;
+            const float4 t = *reinterpret_cast<const float4*>(drow + (ok ? d_pix[q] * p.O + d_o4[q] * 4 : 0));
+            dv[q] = ok ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int q = 0; q < DT_XPL; ++q)
+            if ((x_rc[q] >> 16) != 0x7fff)
+                lx[(x_rc[q] >> 16) * p.rs + (x_rc[q] & 0xffff)] = xv[q];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (d_pix[q] < DT_SEG)
+                *reinterpret_cast<float4*>(ld + d_pix[q] * DT_OMAX + d_o4[q] * 4) = dv[q];
+    };
+
+    if (s_begin < s_end)
+        load(s_begin);
+    for (int it = 0; it < p.segs_per_wave; ++it)   // the same trip count in every wavefront: barriers inside
+    {
+        const int s = s_begin + it;
+        __syncthreads();
+        if (s < s_end)
+            stash();
+        __syncthreads();
+        if (s + 1 < s_end)
+            load(s + 1);
+        if (s < s_end)
+        {
+#pragma unroll 2
+            for (int jj = 0; jj < DT_SEG; jj += 2)
+            {
+                float a[DT_MT], b[DT_NT];
+#pragma unroll
+                for (int mt = 0; mt < DT_MT; ++mt)
+                    a[mt] = lx[a_ptr[mt] + jj * a_step[mt]];
+#pragma unroll
+                for (int nt = 0; nt < DT_NT; ++nt)
+                    b[nt] = lx[b_ptr[nt] + jj * b_step[nt]];
+#pragma unroll
+                for (int mt = 0; mt < DT_MT; ++mt)
+#pragma unroll
+                    for (int nt = 0; nt < DT_NT; ++nt)
+                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mt], b[nt], acc[mt][nt], 0, 0, 0);
+            }
+        }
+    }
+
+    // add the four accumulators in wavefront order; register r of lane l holds element
+    // (m = 8 * (r / 4) + 4 * (l / 32) + r % 4, n = l % 32) of its 32x32 tile
+    __syncthreads();
+    for (int w = 0; w < 4; ++w)
+    {
+        if (wave == w)
+        {
+#pragma unroll
+            for (int mt = 0; mt < DT_MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < DT_NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                    {
+                        const int m = mt * 32 + 8 * (r / 4) + 4 * half + r % 4, n = nt * 32 + l32;
+                        float* dst = lds + m * DT_OMAX + n;
+                        *dst = w == 0 ? acc[mt][nt][r] : *dst + acc[mt][nt][r];
+                    }
+        }
+        __syncthreads();
+    }
+    const int total = p.M * p.O;
+    float* out = p.part + (size_t)blockIdx.x * total;
+    for (int idx = threadIdx.x * 4; idx < total; idx += 256 * 4)
+    {
+        const int m = idx / p.O, n = idx - m * p.O;   // O is a multiple of 4: a quad stays in its row
+        *reinterpret_cast<float4*>(out + idx) = *reinterpret_cast<const float4*>(lds + m * DT_OMAX + n);
+    }
+}
+
 }  // namespace
 
 namespace dh
@@ -375,6 +578,49 @@ int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int 
     }
     prof_end(prof, st);
     DH_LAUNCH_CHECK("dx_few_channels launch");
+    return 0;
+}
+
+
+// Returns 1 when the shape is not one this kernel takes, 0 after a launch (the caller then adds the
+// *splits slices of M x O partial sums at *part), or an error code.
+int conv_dk_thin(const float* x, const float* dy, float** part, int* splits, int N, int H, int W, int C, int Ho, int Wo,
+                 int O, int kh, int kw, int sh, int sw, int pt, int pl, hipStream_t st)
+{
+    const int M = kh * kw * C, row = kw * C;
+    const int rsw = (DT_SEG - 1) * sw * C + row;
+    const int rs = rsw + ((row - rsw) % 32 + 32) % 32;   // rs = row (mod 32): the 32 lanes of a fragment read hit 32 banks
+    if (M > DT_MT * 32 || O > DT_OMAX || O % 4 != 0 || kh * rs > DT_XMAX || kh * rsw > 64 * DT_XPL ||
+        (reinterpret_cast<uintptr_t>(dy) & 15) != 0 || (long)N * Ho * Wo < 2048 || (double)N * H * W * C >= 2147483647.0)
+        return 1;
+    ThinDkParams p{};
+    p.x = x; p.dy = dy;
+    p.N = N; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.O = O; p.kh = kh; p.kw = kw;
+    p.sh = sh; p.sw = sw; p.pt = pt; p.pl = pl;
+    p.M = M; p.row = row; p.rsw = rsw; p.rs = rs;
+    p.segs_per_row = (Wo + DT_SEG - 1) / DT_SEG;
+    const long total = (long)N * Ho * p.segs_per_row;
+    if (total > 0x7fffffffL)
+        return 1;
+    p.total_segs = (int)total;
+    // one workgroup per compute unit (two measured the same: the kernel is bound by the latency of a
+    // segment's load - stage - multiply chain, not by throughput), at least two segments per wavefront
+    long wgs = 1L * num_cus();
+    long per_wave = (total + wgs * 4 - 1) / (wgs * 4);
+    if (per_wave < 2) per_wave = 2;
+    wgs = (total + per_wave * 4 - 1) / (per_wave * 4);
+    p.segs_per_wave = (int)per_wave;
+    p.fd_segs_per_row = FastDiv(p.segs_per_row); p.fd_Ho = FastDiv(Ho); p.fd_rsw = FastDiv(rsw);
+    p.fd_row = FastDiv(row); p.fd_O4 = FastDiv(O / 4);
+    void* ws;
+    DH_TRY(workspace((size_t)wgs * M * O * sizeof(float), &ws, st));
+    p.part = static_cast<float*>(ws);
+    const int prof = prof_begin("dk_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
+    hipLaunchKernelGGL(dk_thin, dim3((unsigned)wgs), dim3(256), 0, st, p);
+    prof_end(prof, st);
+    DH_LAUNCH_CHECK("dk_thin launch");
+    *part = p.part;
+    *splits = (int)wgs;
     return 0;
 }
 

@@ -52,6 +52,12 @@ int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int 
 int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
                   int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st);
 
+// Filter gradient of a thin input (at most 96 filter elements per output channel, at most 64 output
+// channels): writes *splits slices of partial sums to the scratch arena and returns them in *part for
+// the caller to add up; same return convention.
+int conv_dk_thin(const float* x, const float* dy, float** part, int* splits, int N, int H, int W, int C, int Ho, int Wo,
+                 int O, int kh, int kw, int sh, int sw, int pt, int pl, hipStream_t st);
+
 // Test and tuning switches (dh_debug_force_generic_conv, dh_debug_force_splitk).
 extern bool g_force_generic;  // route every convolution through the general kernel
 extern int g_force_splitk;    // > 0: this many k splits (at most one per k-slab) instead of the automatic choice

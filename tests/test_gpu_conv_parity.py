@@ -162,6 +162,36 @@ def test_fwd_from_few_channels(be, orc, shape):
         be.lib.dh_debug_force_generic_conv(0)
 
 
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (2, 64, 64, 3, 5, 5, 64, 2),     # the discriminator's first layer, batch 2
+    (10, 38, 26, 1, 5, 5, 16, 2),    # one channel; 13 output columns: a ragged last segment
+    (4, 70, 37, 2, 3, 3, 48, 2),     # 48 output channels: the second 32-channel tile is partial
+    (4, 40, 40, 4, 4, 4, 32, 1),     # stride 1, even filter, 64 filter elements per output channel
+    (6, 36, 36, 3, 5, 5, 60, 2),     # 60 output channels
+    (4, 48, 40, 4, 5, 4, 8, 2),      # 80 filter elements, 8 output channels
+    (4, 33, 50, 3, 5, 3, 16, 3),     # stride 3: the staged rows do not fit, the implicit GEMM takes it
+])
+def test_dk_from_few_channels(be, orc, shape):
+    """Filter gradient of a thin input (the kernel that reads the gathered operand as a strided view
+    of input rows staged in LDS) against the oracle and against the implicit GEMM, twice for
+    repeatability."""
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(29, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    orc.set_threads(8)
+    exp = orc.conv2d_kernel_grad(dy, x, s, pads)
+    scale = max(1.0, float(np.abs(exp).max()))
+    got = be.conv2d_kernel_grad(dy, x, s, pads)
+    close(got, exp, scale=scale, what="thin filter gradient")
+    np.testing.assert_array_equal(got, be.conv2d_kernel_grad(dy, x, s, pads))
+    be.lib.dh_debug_force_generic_conv(1)
+    try:
+        close(be.conv2d_kernel_grad(dy, x, s, pads), exp, scale=scale, what="implicit GEMM")
+    finally:
+        be.lib.dh_debug_force_generic_conv(0)
+
+
 @pytest.mark.parametrize("generic", [0, 1])
 @pytest.mark.parametrize("shape", [(3, 12, 12, 36, 5, 5, 72, 2), (2, 16, 16, 128, 5, 5, 256, 2), (4, 9, 7, 3, 5, 5, 10, 2)])
 def test_forced_split_counts(be, orc, shape, generic):
