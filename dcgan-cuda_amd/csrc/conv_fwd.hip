@@ -38,6 +38,7 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     if (takes_fast_path(veca, vecb))
     {
         p.skip = p.posmajor = C % BK == 0 && skipping_pays(wgs);
+        order_pixels<MODE_FWD>(p, p.phase, 1, cfg);
         plan_split<MODE_FWD>(p, p.phase, 1, cfg, pair);
     }
     else

@@ -13,11 +13,11 @@ static int same_pad(int n, int k, int s) { int p = n % s == 0 ? k - s : k - n % 
 static long checked = 0;
 
 template <int MODE>
-static bool run(ConvParams& p, const Phase& ph, int bm)
+static bool run(ConvParams& p, const Phase& ph, int bm, int z = 0)
 {
     for (int m0 = 0; m0 < ph.M; m0 += bm)
     {
-        SlabSet s = slab_set<MODE>(p, ph, m0, bm);
+        SlabSet s = slab_set<MODE>(p, ph, m0, bm, z);
         std::set<long> listed;
         SlabIter it; it.seek(s, 0);
         for (int t = 0; t < s.count(); ++t)
@@ -38,7 +38,7 @@ static bool run(ConvParams& p, const Phase& ph, int bm)
                 bool valid; long key;
                 if (MODE == MODE_FWD)
                 {
-                    int pos = m / p.N, i = pos / p.Wo, j = pos % p.Wo;
+                    int pos = pixel_of<MODE_FWD>(p, z, m / p.N), i = pos / p.Wo, j = pos % p.Wo;
                     int tap = k / p.C, c = k % p.C, di = tap / p.kw, dj = tap % p.kw;
                     int ih = i * p.sh + di - p.pt, iw = j * p.sw + dj - p.pl;
                     valid = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
@@ -46,7 +46,7 @@ static bool run(ConvParams& p, const Phase& ph, int bm)
                 }
                 else if (MODE == MODE_DX)
                 {
-                    int pos = m / p.N, hh = pos / ph.Wp, ww = pos % ph.Wp;
+                    int pos = pixel_of<MODE_DX>(p, z, m / p.N), hh = pos / ph.Wp, ww = pos % ph.Wp;
                     int tap = k / p.O, o = k % p.O, th = tap / ph.ntw, tw = tap % ph.ntw;
                     int i = hh + ph.q0h - th, j = ww + ph.q0w - tw;
                     valid = i >= 0 && i < p.Ho && j >= 0 && j < p.Wo;
@@ -72,8 +72,9 @@ static bool run(ConvParams& p, const Phase& ph, int bm)
 
 int main()
 {
-    int fails = 0; long saved = 0, nominal = 0;
+    int fails = 0, permuted = 0; long saved = 0, nominal = 0, saved_perm = 0;
     const int shapes[][8] = { // N H W C O kh sh
+        {64, 16, 16, 16, 16, 5, 2}, {32, 9, 7, 16, 16, 5, 2}, {64, 5, 5, 16, 16, 5, 2}, {32, 6, 6, 16, 16, 3, 1},
         {16, 8, 8, 16, 32, 5, 2}, {32, 8, 8, 32, 16, 5, 2}, {16, 9, 7, 16, 16, 5, 2}, {16, 4, 4, 16, 16, 5, 2}, {16, 6, 6, 16, 16, 3, 1},
         {16, 7, 7, 16, 16, 4, 3}, {64, 8, 8, 32, 16, 5, 2}, {48, 5, 5, 16, 32, 5, 2}, {16, 3, 3, 16, 16, 5, 2}, {16, 2, 2, 16, 16, 5, 2},
         {16, 1, 1, 16, 16, 5, 2}, {3, 8, 8, 16, 16, 5, 2}, {16, 8, 8, 4, 8, 5, 2}, {20, 6, 8, 24, 40, 5, 2}, {16, 16, 16, 16, 16, 5, 2}, {128, 4, 4, 16, 16, 5, 2}};
@@ -86,13 +87,23 @@ int main()
             fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, s, s, pt, pl);
             // FWD
             p.ncols = O; p.phase[0] = Phase{}; p.phase[0].M = N * Ho * Wo; p.phase[0].K = kh * kw * C; p.skip = p.posmajor = C % BK == 0;
+            p.use_perm = 0;
             if (!run<MODE_FWD>(p, p.phase[0], bm)) { ++fails; printf("  FWD shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
-            for (int m0 = 0; m0 < p.phase[0].M; m0 += bm) { saved += slab_set<MODE_FWD>(p, p.phase[0], m0, bm).count(); nominal += (p.phase[0].K + BK - 1) / BK; }
+            order_pixels<MODE_FWD>(p, p.phase, 1, TileCfg{bm, 128});
+            if (p.use_perm)
+            {
+                ++permuted;
+                if (!run<MODE_FWD>(p, p.phase[0], bm)) { ++fails; printf("  FWD (permuted pixels) shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
+                for (int m0 = 0; m0 < p.phase[0].M; m0 += bm) saved_perm += slab_set<MODE_FWD>(p, p.phase[0], m0, bm, 0).count();
+            }
+            p.use_perm = 0;
+            for (int m0 = 0; m0 < p.phase[0].M; m0 += bm) { saved += slab_set<MODE_FWD>(p, p.phase[0], m0, bm, 0).count(); nominal += (p.phase[0].K + BK - 1) / BK; }
             // DK
             p.phase[0].M = kh * kw * C; p.phase[0].K = N * Ho * Wo; p.skip = N % BK == 0;
             if (!run<MODE_DK>(p, p.phase[0], bm)) { ++fails; printf("  DK shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
             // DX phases
             p.ncols = C; p.skip = p.posmajor = O % BK == 0;
+            Phase live[MAX_PHASES]; int nlive = 0;
             for (int q = 0; q < s * s; ++q)
             {
                 Phase f{};
@@ -104,9 +115,21 @@ int main()
                 f.M = N * f.Hp * f.Wp; f.K = f.nth * f.ntw * O;
                 f.fd_HpWp = FastDiv(f.Hp * f.Wp); f.fd_Wp = FastDiv(f.Wp); f.fd_ntw = FastDiv(f.ntw > 0 ? f.ntw : 1);
                 if (f.K == 0) continue;
+                p.use_perm = 0;
                 if (!run<MODE_DX>(p, f, bm)) { ++fails; printf("  DX shape N%d H%d W%d C%d O%d k%d s%d bm%d phase %d\n", N, H, W, C, O, kh, s, bm, q); }
+                if (nlive < MAX_PHASES) live[nlive++] = f;
             }
+            order_pixels<MODE_DX>(p, live, nlive, TileCfg{bm, 128});
+            if (p.use_perm)
+            {
+                ++permuted;
+                for (int z = 0; z < nlive; ++z)
+                    if (!run<MODE_DX>(p, live[z], bm, z)) { ++fails; printf("  DX (permuted pixels) shape N%d H%d W%d C%d O%d k%d s%d bm%d slot %d\n", N, H, W, C, O, kh, s, bm, z); }
+            }
+            p.use_perm = 0;
         }
-    printf("%ld element checks, %d failures; FWD slabs kept %ld of %ld\n", checked, fails, saved, nominal);
+    printf("%ld element checks, %d failures; FWD slabs kept %ld of %ld; %d launches with permuted pixels (FWD slabs kept %ld)\n",
+           checked, fails, saved, nominal, permuted, saved_perm);
+    if (permuted == 0) { printf("no shape exercised the permuted pixel order\n"); return 1; }
     return fails != 0;
 }

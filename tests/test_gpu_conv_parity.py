@@ -242,6 +242,10 @@ def test_forced_split_counts(be, orc, shape, generic):
     (16, 2, 2, 16, 5, 5, 16, 2),     # a single output pixel
     (16, 1, 1, 16, 5, 5, 16, 2),     # 1x1 image: one live tap
     (256, 4, 4, 16, 5, 5, 16, 2),    # two row tiles per pixel
+    (64, 8, 8, 16, 5, 5, 32, 2),     # two pixels per tile: pixels taken in the order sorted by their tap box
+    (64, 5, 5, 16, 5, 5, 16, 2),     # ... with an odd number of pixels
+    (64, 16, 16, 16, 5, 5, 16, 2),   # ... 64 pixels per stride phase (the most the pixel table holds)
+    (64, 6, 6, 16, 3, 3, 16, 1),     # ... stride 1
 ])
 @pytest.mark.parametrize("splits", [0, 5])
 def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
