@@ -219,7 +219,13 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     if (m > 0x7fffffff || n > 0x7fffffff || p > 0x7fffffff) return fail(DH_EINVAL, "%s: extent too large", who);
     hipStream_t st = as_stream(stream);
     ProfScope prof("dense gemm", 2.0 * m * n * p, st);
-    if (n <= SK_MAXK && sbj == 1 && p >= 64 && m > 4)
+    if (n <= SK_MAXK && sbj == 1 && p >= 64 && m > 4 && ((p + 63) / 64) * ((m + 63) / 64) < 2 * (size_t)num_cus())
+    {
+        // too few workgroups of 64 rows to fill the device: 16 rows each
+        hipLaunchKernelGGL(gemm_skinny<4>, dim3((unsigned)((p + 63) / 64), (unsigned)((m + 15) / 16)), dim3(256), 0, st, a, b,
+                           bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+    }
+    else if (n <= SK_MAXK && sbj == 1 && p >= 64 && m > 4)
         hipLaunchKernelGGL(gemm_skinny<16>, dim3((unsigned)((p + 63) / 64), (unsigned)((m + 63) / 64)), dim3(256), 0, st, a, b,
                            bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
     else if (n <= SK_MAXK && sbj == 1 && p >= 64)
