@@ -443,7 +443,9 @@ __global__ __launch_bounds__(256) void dk_thin(const ThinDkParams p)
             load(s + 1);
         if (s < s_end)
         {
-#pragma unroll 2
+            // fully unrolled: the LDS reads of all eight steps are issued ahead of the MFMAs (340 registers,
+            // one wavefront per SIMD -- which is all the launch has anyway)
+#pragma unroll
             for (int jj = 0; jj < DT_SEG; jj += 2)
             {
                 float a[DT_MT], b[DT_NT];
