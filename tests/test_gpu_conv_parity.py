@@ -283,6 +283,29 @@ def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
         be.lib.dh_debug_force_splitk(0)
 
 
+def test_split_with_more_workgroups_than_the_table_holds(be, orc):
+    """40 row tiles cut into 25 splits each are more workgroups than the kernel's workgroup table
+    lists (640): the launch falls back to the nested grid in which every tile uses all its splits."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    shape = (80, 16, 16, 16, 5, 5, 16, 2)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(37, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    orc.set_threads(8)
+    exp_f = orc.relu_leaky(orc.bias_add(orc.conv2d(x, k, (s, s)), bias), 0.2)
+    exp_x = orc.conv2d_input_grad(dy, k, s, (H, W))
+    exp_k = orc.conv2d_kernel_grad(dy, x, s, pads)
+    be.lib.dh_debug_force_splitk(25)
+    try:
+        close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), exp_f, what="fwd")
+        close(be.conv2d_input_grad(dy, k, s, (H, W)), exp_x, what="dx")
+        close(be.conv2d_kernel_grad(dy, x, s, pads), exp_k, scale=max(1.0, float(np.abs(exp_k).max())), what="dk")
+    finally:
+        be.lib.dh_debug_force_splitk(0)
+
+
 @pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
     (3, 12, 12, 36, 5, 5, 72, 2),     # partial tiles in m, n and k
     (2, 32, 32, 64, 5, 5, 128, 2),    # D1 at batch 2
