@@ -25,8 +25,7 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
             if (blocks > 4096) blocks = 4096;
             ProfScope prof("hbm:splitk_reduce (4 B x (splits + 1) per output)", 4.0 * n * (splits + 1), as_stream(stream));
             hipLaunchKernelGGL(splitk_reduce_wide, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), part, dk,
-                               (float*)nullptr, (const float*)nullptr, n, n, O, splits, (int)DH_ACT_NONE, 0.f,
-                               (const float*)nullptr, (const float*)nullptr, (int)DH_ACT_NONE, 0.f);
+                               (float*)nullptr, (const float*)nullptr, n, n, O, splits, (int)DH_ACT_NONE, 0.f);
             DH_LAUNCH_CHECK("splitk_reduce_wide launch");
             return 0;
         }

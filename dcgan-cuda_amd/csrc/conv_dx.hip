@@ -9,15 +9,13 @@ namespace
 // One instance (dy2 == dx2 == nullptr) or two instances that share the filter.
 int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, float* dx, float* dx2, int N, int Ho,
             int Wo, int O, int kh, int kw, int C, int sh, int sw, int pad_top, int pad_left, int H, int W,
-            const float* bias, int act, float alpha, void* stream, const float* gate = nullptr,
-            const float* gate2 = nullptr, int gate_act = DH_ACT_NONE, float gate_alpha = 0.f)
+            const float* bias, int act, float alpha, void* stream)
 {
     DH_TRY(ensure_init());
     DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     const bool pair = dy2 != nullptr || dx2 != nullptr;
     if (!dy || !k || !dx || (pair && (!dy2 || !dx2))) return fail(DH_EINVAL, "%s: null tensor", who);
-    if (gate && pair && !gate2) return fail(DH_EINVAL, "%s: a gate for each instance", who);
-    if (!pair && !g_force_generic && !gate)
+    if (!pair && !g_force_generic)
     {
         const int rc = conv_dx_few_channels(dy, k, dx, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias,
                                             act, alpha, as_stream(stream));
@@ -28,7 +26,6 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = dy; p.b_src = k; p.out = dx; p.bias = bias; p.act = act; p.alpha = alpha;
     p.a_src2 = dy2; p.out2 = dx2;
-    p.gate = gate; p.gate2 = gate2; p.gate_act = gate_act; p.gate_alpha = gate_alpha;
     p.ncols = C;
     p.out_elems = (size_t)N * H * W * C;
 
@@ -118,17 +115,6 @@ int dh_conv2d_dx(const float* dy, const float* k, float* dx, int N, int Ho, int 
 {
     return conv_dx("dh_conv2d_dx", dy, nullptr, k, dx, nullptr, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W,
                    bias, act, alpha, stream);
-}
-
-int dh_conv2d_dx_gated(const float* dy1, const float* dy2, const float* k, float* dx1, float* dx2, int N, int Ho,
-                       int Wo, int O, int kh, int kw, int C, int sh, int sw, int pad_top, int pad_left, int H, int W,
-                       const float* gate1, const float* gate2, int gate_act, float gate_alpha, void* stream)
-{
-    if (!gate1) return fail(DH_EINVAL, "dh_conv2d_dx_gated: null gate");
-    if ((dy2 != nullptr) != (dx2 != nullptr) || (dy2 != nullptr) != (gate2 != nullptr))
-        return fail(DH_EINVAL, "dh_conv2d_dx_gated: the second instance needs dy2, dx2 and gate2");
-    return conv_dx("dh_conv2d_dx_gated", dy1, dy2, k, dx1, dx2, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W,
-                   nullptr, DH_ACT_NONE, 0.f, stream, gate1, gate2, gate_act, gate_alpha);
 }
 
 int dh_conv2d_dx_pair(const float* dy1, const float* dy2, const float* k, float* dx1, float* dx2, int N, int Ho,

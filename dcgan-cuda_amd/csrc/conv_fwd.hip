@@ -6,15 +6,13 @@ namespace
 // One instance (x2 == y2 == nullptr) or two instances that share the filter.
 int conv_fwd(const char* who, const float* x, const float* x2, const float* k, float* y, float* y2, int N, int H, int W,
              int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo, const float* bias,
-             int act, float alpha, void* stream, const float* gate = nullptr, const float* gate2 = nullptr,
-             int gate_act = DH_ACT_NONE, float gate_alpha = 0.f)
+             int act, float alpha, void* stream)
 {
     DH_TRY(ensure_init());
     DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     const bool pair = x2 != nullptr || y2 != nullptr;
     if (!x || !k || !y || (pair && (!x2 || !y2))) return fail(DH_EINVAL, "%s: null tensor", who);
-    if (gate && pair && !gate2) return fail(DH_EINVAL, "%s: a gate for each instance", who);
-    if (!pair && !g_force_generic && !gate)
+    if (!pair && !g_force_generic)
     {
         const int rc = conv_fwd_thin(x, k, y, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias, act, alpha,
                                      as_stream(stream));
@@ -25,7 +23,6 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left);
     p.a_src = x; p.b_src = k; p.out = y; p.bias = bias; p.act = act; p.alpha = alpha;
     p.a_src2 = x2; p.out2 = y2;
-    p.gate = gate; p.gate2 = gate2; p.gate_act = gate_act; p.gate_alpha = gate_alpha;
     p.ncols = O;
     p.out_elems = (size_t)N * Ho * Wo * O;
     p.phase[0].M = N * Ho * Wo;
@@ -66,17 +63,6 @@ int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W,
 {
     return conv_fwd("dh_conv2d_fwd", x, nullptr, k, y, nullptr, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo,
                     bias, act, alpha, stream);
-}
-
-int dh_conv2d_fwd_gated(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
-                        int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,
-                        const float* gate1, const float* gate2, int gate_act, float gate_alpha, void* stream)
-{
-    if (!gate1) return fail(DH_EINVAL, "dh_conv2d_fwd_gated: null gate");
-    if ((x2 != nullptr) != (y2 != nullptr) || (x2 != nullptr) != (gate2 != nullptr))
-        return fail(DH_EINVAL, "dh_conv2d_fwd_gated: the second instance needs x2, y2 and gate2");
-    return conv_fwd("dh_conv2d_fwd_gated", x1, x2, k, y1, y2, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo,
-                    nullptr, DH_ACT_NONE, 0.f, stream, gate1, gate2, gate_act, gate_alpha);
 }
 
 int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,

@@ -50,8 +50,6 @@ _SIGS = {
     "dh_conv2d_fwd_pair": [_vp] * 5 + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dx_pair": [_vp] * 5 + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dk_pair": [_vp] * 5 + [_i] * 13 + [_vp],
-    "dh_conv2d_fwd_gated": [_vp] * 5 + [_i] * 13 + [_vp, _vp, _i, _f, _vp],
-    "dh_conv2d_dx_gated": [_vp] * 5 + [_i] * 13 + [_vp, _vp, _i, _f, _vp],
     "dh_bias_add": [_vp, _vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad": [_vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad_parts": [_vp, _vp, _sz, _sz, _vp],
@@ -296,38 +294,6 @@ class HipBackend:
         check(self.lib.dh_conv2d_dk_pair(a1.ptr, b1.ptr, a2.ptr, b2.ptr, out.ptr, N, H, W, Cc, Ho, Wo, O, kh, kw,
                                          stride, stride, pads[0] // 2, pads[1] // 2, self.stream))
         return out.numpy()
-
-    def conv2d_input_grad_gated(self, dy, k, stride, in_hw, gate, gate_act, gate_alpha=0.0, dy2=None, gate2=None):
-        """act'(gate) * dx(dy, k); with dy2 / gate2 the paired launch, returning both results."""
-        N, Ho, Wo, O = dy.shape
-        kh, kw, Cc, O2 = k.shape
-        H, W = in_hw
-        pads = (same_pad(H, kh, stride)[0], same_pad(W, kw, stride)[0])
-        ddy, dk, dg = self._up(dy, k, gate)
-        dx = Buf((N, H, W, Cc))
-        ddy2 = Buf.from_numpy(dy2) if dy2 is not None else None
-        dg2 = Buf.from_numpy(gate2) if gate2 is not None else None
-        dx2 = Buf((N, H, W, Cc)) if dy2 is not None else None
-        check(self.lib.dh_conv2d_dx_gated(ddy.ptr, ddy2.ptr if ddy2 else None, dk.ptr, dx.ptr, dx2.ptr if dx2 else None,
-                                          N, Ho, Wo, O, kh, kw, Cc, stride, stride, pads[0] // 2, pads[1] // 2, H, W,
-                                          dg.ptr, dg2.ptr if dg2 else None, gate_act, gate_alpha, self.stream))
-        return (dx.numpy(), dx2.numpy()) if dx2 else dx.numpy()
-
-    def conv2d_gated(self, x, k, strides, gate, gate_act, gate_alpha=0.0, x2=None, gate2=None):
-        """act'(gate) * conv(x, k) (the input gradient of a transposed convolution); optionally paired."""
-        N, H, W, Cc = x.shape
-        kh, kw, C2, O = k.shape
-        pads = (same_pad(H, kh, strides[0])[0], same_pad(W, kw, strides[1])[0])
-        Ho, Wo = -(-H // strides[0]), -(-W // strides[1])
-        dx, dk, dg = self._up(x, k, gate)
-        y = Buf((N, Ho, Wo, O))
-        dx2 = Buf.from_numpy(x2) if x2 is not None else None
-        dg2 = Buf.from_numpy(gate2) if gate2 is not None else None
-        y2 = Buf((N, Ho, Wo, O)) if x2 is not None else None
-        check(self.lib.dh_conv2d_fwd_gated(dx.ptr, dx2.ptr if dx2 else None, dk.ptr, y.ptr, y2.ptr if y2 else None,
-                                           N, H, W, Cc, kh, kw, O, strides[0], strides[1], pads[0] // 2, pads[1] // 2,
-                                           Ho, Wo, dg.ptr, dg2.ptr if dg2 else None, gate_act, gate_alpha, self.stream))
-        return (y.numpy(), y2.numpy()) if y2 else y.numpy()
 
     def conv2d_input_grad(self, dy, k, stride, in_hw, bias=None, act=ACT_NONE, alpha=0.0):
         N, Ho, Wo, O = dy.shape

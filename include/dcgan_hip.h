@@ -152,21 +152,6 @@ int dh_conv2d_dk_pair(const float* x1, const float* dy1, const float* x2, const 
                       int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left,
                       void* stream);
 
-/* Input gradients whose result is multiplied by an activation's derivative in the write-out:
- *   dh_conv2d_dx_gated:  dx1 = act'(gate1) * dx(dy1, k)   (conv2d_input_grad followed by relu_grad /
- *                        leaky_relu_grad / tanh_grad / sigmoid_grad, src/ops/graph.cu backward lists)
- *   dh_conv2d_fwd_gated: y1 = act'(gate1) * conv(x1, k)   (conv2d_transpose_input_grad followed by the same)
- * gate is the tensor the activation-gradient operator reads (dh_relu_grad ... dh_sigmoid_grad: z, or the
- * forward output), gate_act one of DH_ACT_*.  The unactivated gradient is never written, which saves the
- * activation-gradient pass over it.  With x2 / y2 / gate2 (dy2 / dx2 / gate2) not null the call is a paired
- * launch as above, otherwise pass all three as NULL.  No bias, no activation besides the gate. */
-int dh_conv2d_fwd_gated(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
-                        int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,
-                        const float* gate1, const float* gate2, int gate_act, float gate_alpha, void* stream);
-int dh_conv2d_dx_gated(const float* dy1, const float* dy2, const float* k, float* dx1, float* dx2, int N, int Ho,
-                       int Wo, int O, int kh, int kw, int C, int sh, int sw, int pad_top, int pad_left, int H, int W,
-                       const float* gate1, const float* gate2, int gate_act, float gate_alpha, void* stream);
-
 /* ---- bias and activations: coalesced, vectorised, one pass over HBM ----------------------------- */
 
 /* out[r,c] = z[r,c] + b[c].  conv2d_bias_add lowers to this (src/ops/conv2d-bias-add.cu:35-38);

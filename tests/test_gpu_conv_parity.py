@@ -283,51 +283,6 @@ def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
         be.lib.dh_debug_force_splitk(0)
 
 
-@pytest.mark.parametrize("generic", [0, 1])
-@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
-    (3, 12, 12, 36, 5, 5, 72, 2),     # partial tiles
-    (4, 8, 8, 256, 5, 5, 512, 2),     # split contraction
-    (64, 8, 8, 16, 5, 5, 32, 2),      # permuted pixel order
-    (2, 9, 7, 6, 3, 3, 10, 1),        # channel counts not divisible by 4: element-wise write-out
-])
-def test_gated_input_gradients(be, orc, shape, generic):
-    """Input gradient (and forward product, the input gradient of a transposed convolution) with the
-    activation gradient applied in the write-out: equal to the two separate operators -- to the bit
-    for relu and leaky relu, whose gate is a selection -- single, paired and with a forced split."""
-    import __graft_entry__ as ge
-    A = ge.load_package().hipabi
-    print("shape", shape, "generic", generic, flush=True)
-    N, H, W, C, kh, kw, O, s = shape
-    x, k, dy = rand_conv_inputs(51, *shape)
-    x2, _, dy2 = rand_conv_inputs(52, *shape)
-    rng = np.random.default_rng(53)
-    zx = rng.uniform(-1, 1, x.shape).astype(np.float32)    # pre-activation values at the convolution's input
-    zx2 = rng.uniform(-1, 1, x.shape).astype(np.float32)
-    zy = rng.uniform(-1, 1, dy.shape).astype(np.float32)   # ... and at its output
-    be.lib.dh_debug_force_generic_conv(generic)
-    try:
-        for splits in (0, 3):
-            be.lib.dh_debug_force_splitk(splits)
-            plain = be.conv2d_input_grad(dy, k, s, (H, W))
-            np.testing.assert_array_equal(be.conv2d_input_grad_gated(dy, k, s, (H, W), zx, A.ACT_LEAKY, 0.2),
-                                          be.leaky_relu_grad(zx, plain, 0.2))
-            np.testing.assert_array_equal(be.conv2d_input_grad_gated(dy, k, s, (H, W), zx, A.ACT_RELU),
-                                          be.relu_grad(zx, plain))
-            t = np.tanh(zx)
-            close(be.conv2d_input_grad_gated(dy, k, s, (H, W), t, A.ACT_TANH), be.tanh_grad(t, plain), what="tanh gate")
-            fwd = be.conv2d(x, k, (s, s))
-            np.testing.assert_array_equal(be.conv2d_gated(x, k, (s, s), zy, A.ACT_RELU), be.relu_grad(zy, fwd))
-            if not generic and C % 4 == 0 and O % 4 == 0:
-                g1, g2 = be.conv2d_input_grad_gated(dy, k, s, (H, W), zx, A.ACT_LEAKY, 0.2, dy2=dy2, gate2=zx2)
-                p1, p2 = be.conv2d_input_grad_pair(dy, dy2, k, s, (H, W))
-                np.testing.assert_array_equal(g1, be.leaky_relu_grad(zx, p1, 0.2))
-                np.testing.assert_array_equal(g2, be.leaky_relu_grad(zx2, p2, 0.2))
-    finally:
-        be.lib.dh_debug_force_splitk(0)
-        be.lib.dh_debug_force_generic_conv(0)
-    close(plain, orc.conv2d_input_grad(dy, k, s, (H, W)), what="dx")
-
-
 def test_split_with_more_workgroups_than_the_table_holds(be, orc):
     """40 row tiles cut into 25 splits each are more workgroups than the kernel's workgroup table
     lists (640): the launch falls back to the nested grid in which every tile uses all its splits."""
