@@ -42,7 +42,7 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
     p.phase[0].K = N * Ho * Wo;
     const bool veca = C % 4 == 0 && aligned16(x) && aligned16(x2);
     const bool vecb = O % 4 == 0 && aligned16(dy) && aligned16(dy2);
-    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)N * Ho * Wo * O * 4};
+    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)N * Ho * Wo * O * 4, true};
     if (pair && !takes_fast_path(veca, vecb))
         return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const long slabs_one = (p.phase[0].K + BK - 1) / BK;

@@ -68,16 +68,16 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     std::reverse(all + (n_live + 1) / 2, all + n_live);
     const bool veca = O % 4 == 0 && aligned16(dy) && aligned16(dy2);
     const bool vecb = O % 4 == 0 && aligned16(k);
-    g_operand_bytes = {(size_t)N * Ho * Wo * O * 4, (size_t)kh * kw * C * O * 4};
+    g_operand_bytes = {(size_t)N * Ho * Wo * O * 4, (size_t)kh * kw * C * O * 4, O % BK == 0};
     if (pair && (!takes_fast_path(veca, vecb) || C % 4 != 0))
-        return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
+        return fail(DH_ENOTSUP, "%s: the paired launch needs dy channels divisible by 16, result channels divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const int instances = pair ? 2 : 1;
     const TileCfg cfg = pick_tile(max_m, C);
     for (int q = 0; q < n_live; ++q)
         total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;
     if (takes_fast_path(veca, vecb))
     {
-        p.skip = p.posmajor = O % BK == 0 && skipping_pays(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances);
+        p.skip = p.posmajor = skipping_pays(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances);
         order_pixels<MODE_DX>(p, all, n_live, cfg);
         plan_split<MODE_DX>(p, all, n_live, cfg, pair);
     }

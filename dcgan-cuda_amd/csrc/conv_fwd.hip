@@ -29,15 +29,15 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     p.phase[0].K = kh * kw * C;
     const bool veca = C % 4 == 0 && aligned16(x) && aligned16(x2);
     const bool vecb = O % 4 == 0 && aligned16(k);
-    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)kh * kw * C * O * 4};
+    g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)kh * kw * C * O * 4, C % BK == 0};
     if (pair && !takes_fast_path(veca, vecb))
-        return fail(DH_ENOTSUP, "%s: the paired launch needs channel counts divisible by 4, 16-byte aligned tensors below 2 GiB", who);
+        return fail(DH_ENOTSUP, "%s: the paired launch needs input channels divisible by 16, output channels divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const TileCfg cfg = pick_tile(p.phase[0].M, O);
     const int instances = pair ? 2 : 1;
     const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
     if (takes_fast_path(veca, vecb))
     {
-        p.skip = p.posmajor = C % BK == 0 && skipping_pays(wgs);
+        p.skip = p.posmajor = skipping_pays(wgs);
         order_pixels<MODE_FWD>(p, p.phase, 1, cfg);
         plan_split<MODE_FWD>(p, p.phase, 1, cfg, pair);
     }

@@ -472,7 +472,9 @@ bool pairable(const ConvCall& c)
     auto aligned = [](const void* q) { return (reinterpret_cast<std::uintptr_t>(q) & 15) == 0; };
     const double in_bytes = 4.0 * g.N * g.H * g.W * g.C, out_bytes = 4.0 * g.N * g.Ho * g.Wo * g.O;
     const double k_bytes = 4.0 * g.kh * g.kw * g.C * g.O, lim = 2147483648.0;
-    return g.C % 4 == 0 && g.O % 4 == 0 && in_bytes < lim && out_bytes < lim && k_bytes < lim && aligned(c.a) &&
+    // the paired launches need the buffer-load kernel, whose k-slabs of 16 must not straddle filter taps
+    const bool tapwise = c.kind == 0 ? g.C % 16 == 0 : c.kind == 1 ? g.O % 16 == 0 : true;
+    return tapwise && g.C % 4 == 0 && g.O % 4 == 0 && in_bytes < lim && out_bytes < lim && k_bytes < lim && aligned(c.a) &&
            aligned(c.b) && aligned(c.out) && aligned(c.bias);
 }
 

@@ -139,8 +139,9 @@ int dh_conv2d_dk(const float* x, const float* dy, float* dk,
  *   dh_conv2d_dx_pair:  dx1 = dx(dy1, k), dx2 = dx(dy2, k)           (+ the same bias / activation)
  *   dh_conv2d_dk_pair:  dk = dk(x1, dy1) + dk(x2, dy2), the sum the reference forms with an `add`
  *                       node when a filter receives gradient along two paths (src/ops/graph.cu:295-308)
- * They need the 16-byte buffer-load kernel (channel counts divisible by 4, 16-byte aligned tensors
- * below 2 GiB) and return DH_ENOTSUP otherwise; results agree with the single calls to rounding
+ * They need the buffer-load kernel (channel counts divisible by 4 and, for the channels the product
+ * contracts over -- the input's for fwd, dy's for dx -- by 16; 16-byte aligned tensors below 2 GiB)
+ * and return DH_ENOTSUP otherwise; results agree with the single calls to rounding
  * (the contraction may be split differently). */
 int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
                        int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,

@@ -38,19 +38,19 @@ static bool run(ConvParams& p, const Phase& ph, int bm, int z = 0)
                 bool valid; long key;
                 if (MODE == MODE_FWD)
                 {
-                    int pos = pixel_of<MODE_FWD>(p, z, m / p.N), i = pos / p.Wo, j = pos % p.Wo;
+                    int pos = p.posmajor ? pixel_of<MODE_FWD>(p, z, m / p.N) : m % (p.Ho * p.Wo), i = pos / p.Wo, j = pos % p.Wo;
                     int tap = k / p.C, c = k % p.C, di = tap / p.kw, dj = tap % p.kw;
                     int ih = i * p.sh + di - p.pt, iw = j * p.sw + dj - p.pl;
                     valid = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-                    key = p.skip ? ((long)di * 100000 + dj) * 100000 + c / BK : k / BK;
+                    key = ((long)di * 100000 + dj) * 100000 + c / BK;   // the kernel's slabs never straddle taps
                 }
                 else if (MODE == MODE_DX)
                 {
-                    int pos = pixel_of<MODE_DX>(p, z, m / p.N), hh = pos / ph.Wp, ww = pos % ph.Wp;
+                    int pos = p.posmajor ? pixel_of<MODE_DX>(p, z, m / p.N) : m % (ph.Hp * ph.Wp), hh = pos / ph.Wp, ww = pos % ph.Wp;
                     int tap = k / p.O, o = k % p.O, th = tap / ph.ntw, tw = tap % ph.ntw;
                     int i = hh + ph.q0h - th, j = ww + ph.q0w - tw;
                     valid = i >= 0 && i < p.Ho && j >= 0 && j < p.Wo;
-                    key = p.skip ? ((long)th * 100000 + tw) * 100000 + o / BK : k / BK;
+                    key = ((long)th * 100000 + tw) * 100000 + o / BK;
                 }
                 else
                 {
@@ -86,9 +86,11 @@ int main()
             ConvParams p{};
             fill_common(p, N, H, W, C, Ho, Wo, O, kh, kw, s, s, pt, pl);
             // FWD
-            p.ncols = O; p.phase[0] = Phase{}; p.phase[0].M = N * Ho * Wo; p.phase[0].K = kh * kw * C; p.skip = p.posmajor = C % BK == 0;
+            p.ncols = O; p.phase[0] = Phase{}; p.phase[0].M = N * Ho * Wo; p.phase[0].K = kh * kw * C; p.skip = p.posmajor = 0;
             p.use_perm = 0;
-            if (!run<MODE_FWD>(p, p.phase[0], bm)) { ++fails; printf("  FWD shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
+            if (C % BK == 0 && !run<MODE_FWD>(p, p.phase[0], bm)) { ++fails; printf("  FWD (nothing skipped) shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
+            p.skip = p.posmajor = C % BK == 0;
+            if (p.skip && !run<MODE_FWD>(p, p.phase[0], bm)) { ++fails; printf("  FWD shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
             order_pixels<MODE_FWD>(p, p.phase, 1, TileCfg{bm, 128});
             if (p.use_perm)
             {
@@ -97,7 +99,7 @@ int main()
                 for (int m0 = 0; m0 < p.phase[0].M; m0 += bm) saved_perm += slab_set<MODE_FWD>(p, p.phase[0], m0, bm, 0).count();
             }
             p.use_perm = 0;
-            for (int m0 = 0; m0 < p.phase[0].M; m0 += bm) { saved += slab_set<MODE_FWD>(p, p.phase[0], m0, bm, 0).count(); nominal += (p.phase[0].K + BK - 1) / BK; }
+            if (p.skip) for (int m0 = 0; m0 < p.phase[0].M; m0 += bm) { saved += slab_set<MODE_FWD>(p, p.phase[0], m0, bm, 0).count(); nominal += (p.phase[0].K + BK - 1) / BK; }
             // DK
             p.phase[0].M = kh * kw * C; p.phase[0].K = N * Ho * Wo; p.skip = N % BK == 0;
             if (!run<MODE_DK>(p, p.phase[0], bm)) { ++fails; printf("  DK shape N%d H%d W%d C%d O%d k%d s%d bm%d\n", N, H, W, C, O, kh, s, bm); }
@@ -116,6 +118,10 @@ int main()
                 f.fd_HpWp = FastDiv(f.Hp * f.Wp); f.fd_Wp = FastDiv(f.Wp); f.fd_ntw = FastDiv(f.ntw > 0 ? f.ntw : 1);
                 if (f.K == 0) continue;
                 p.use_perm = 0;
+                if (O % BK != 0) continue;
+                p.skip = p.posmajor = 0;
+                if (!run<MODE_DX>(p, f, bm)) { ++fails; printf("  DX (nothing skipped) shape N%d H%d W%d C%d O%d k%d s%d bm%d phase %d\n", N, H, W, C, O, kh, s, bm, q); }
+                p.skip = p.posmajor = 1;
                 if (!run<MODE_DX>(p, f, bm)) { ++fails; printf("  DX shape N%d H%d W%d C%d O%d k%d s%d bm%d phase %d\n", N, H, W, C, O, kh, s, bm, q); }
                 if (nlive < MAX_PHASES) live[nlive++] = f;
             }

@@ -307,10 +307,10 @@ def test_split_with_more_workgroups_than_the_table_holds(be, orc):
 
 
 @pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
-    (3, 12, 12, 36, 5, 5, 72, 2),     # partial tiles in m, n and k
+    (3, 12, 12, 48, 5, 5, 80, 2),     # partial tiles in m and n
     (2, 32, 32, 64, 5, 5, 128, 2),    # D1 at batch 2
     (4, 8, 8, 256, 5, 5, 512, 2),     # D3 at batch 4 (split-K)
-    (2, 9, 7, 8, 3, 3, 12, 1),        # stride 1, contraction of one instance not a multiple of 16
+    (2, 9, 7, 16, 3, 3, 32, 1),       # stride 1, odd extents
 ])
 def test_paired_launches(be, orc, shape):
     """Two instances of a product in one launch (same filter, two sets of activations): forward and
@@ -367,7 +367,8 @@ def test_paired_launches_at_batch_64_match_the_single_launches(be, shape):
 
 
 def test_paired_launch_refuses_what_it_cannot_take(be):
-    """Channel counts that are not multiples of 4 have no paired kernel: DH_ENOTSUP, not a wrong result."""
+    """Channel counts that are not multiples of 4 -- or, for the channels a forward / input-gradient
+    product contracts over, of 16 -- have no paired kernel: DH_ENOTSUP, not a wrong result."""
     import __graft_entry__ as ge
     A = ge.load_package().hipabi
     x, k, dy = rand_conv_inputs(1, 2, 8, 8, 3, 5, 5, 6, 2)
@@ -375,6 +376,11 @@ def test_paired_launch_refuses_what_it_cannot_take(be):
         be.conv2d_pair(x, x, k, (2, 2))
     with pytest.raises(A.HipError, match="10002"):
         be.conv2d_kernel_grad_pair(dy, x, dy, x, 2, (3, 3))
+    x, k, dy = rand_conv_inputs(1, 2, 8, 8, 36, 5, 5, 72, 2)
+    with pytest.raises(A.HipError, match="10002"):
+        be.conv2d_pair(x, x, k, (2, 2))
+    with pytest.raises(A.HipError, match="10002"):
+        be.conv2d_input_grad_pair(dy, dy, k, 2, (8, 8))
 
 
 def test_dk_is_reproducible(be):
