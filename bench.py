@@ -43,12 +43,12 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # summaries are kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
     # launch-weighted over the single and the paired instantiation of a tag
-    "conv_igemm_fast<fwd,128x128>": 131.8e6,    # 6 single launches of 100.8 MB, 3 paired of 193.9 MB per iteration
-    "conv_igemm_fast<dx,128x128>": 128.0e6,     # 6 x 114.9 MB, 2 x 167.1 MB
-    "conv_igemm_fast<dk,128x128>": 192.2e6,     # 3 x 126.1 MB, 3 x 258.2 MB
-    "conv_igemm_fast<dx,128x64>": 65.5e6,       # 3 x 34.0 MB, 1 x 160.0 MB
+    "conv_igemm_fast<fwd,128x128>": 133.6e6,    # 6 single launches of 102.3 MB, 3 paired of 196.1 MB per iteration
+    "conv_igemm_fast<dx,128x128>": 125.5e6,     # 6 x 112.2 MB, 2 x 165.7 MB
+    "conv_igemm_fast<dk,128x128>": 191.3e6,     # 3 x 126.2 MB, 3 x 256.4 MB
+    "conv_igemm_fast<dx,128x64>": 55.0e6,       # 3 x 35.9 MB, 1 x 112.1 MB
     "fwd_thin": 21.7e6,
-    "dk_thin": 25.5e6,
+    "dk_thin": 25.6e6,
     "dx_few_channels": 27.2e6,
 }
 
