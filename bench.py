@@ -43,10 +43,11 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # summaries are kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
     # launch-weighted over the single and the paired instantiation of a tag
-    "conv_igemm_fast<fwd,128x128>": 133.6e6,    # 6 single launches of 102.3 MB, 3 paired of 196.1 MB per iteration
-    "conv_igemm_fast<dx,128x128>": 125.5e6,     # 6 x 112.2 MB, 2 x 165.7 MB
-    "conv_igemm_fast<dk,128x128>": 191.3e6,     # 3 x 126.2 MB, 3 x 256.4 MB
-    "conv_igemm_fast<dx,128x64>": 55.0e6,       # 3 x 35.9 MB, 1 x 112.1 MB
+    "conv_igemm_fast<dx,128x64>": 87.3e6,       # 9 single launches of 71.6 MB, 2 paired of 157.5 MB per iteration
+    "conv_igemm_fast<fwd,128x64>": 135.2e6,     # 6 x 119.9 MB, 1 x 226.5 MB
+    "conv_igemm_fast<dk,128x128>": 191.4e6,     # 3 x 126.0 MB, 3 x 256.8 MB
+    "conv_igemm_fast<fwd,128x128>": 182.1e6,    # 2 paired
+    "conv_igemm_fast<dx,128x128>": 172.5e6,     # 1 paired
     "fwd_thin": 21.7e6,
     "dk_thin": 25.6e6,
     "dx_few_channels": 27.2e6,
@@ -90,15 +91,15 @@ def synthetic(batch, seed=1234):
 
 def cpu_baseline(batch, budget_s=25.0):
     """Times the reference's CPU operators (compiled from its own header into oracle/_ref) on one
-    core: conv2d, conv2d_input_grad, conv2d_kernel_grad on layer D1 at batch 1 (and D0 for the
-    cheap forward), then extrapolates one iteration from the measured FLOP/s of each class."""
+    core: conv2d, conv2d_input_grad, conv2d_kernel_grad on layer D1 at batch 8 (about 10 s of CPU
+    work), then extrapolates one iteration from the measured FLOP/s of each class."""
     oracle = ge.load_oracle()
     kind = "reference" if oracle.have_ref() else "port"
     orc = oracle.Oracle("ref" if kind == "reference" else "orc")
     orc.set_threads(1)
     rng = np.random.default_rng(0)
     H, W, C, O = LAYERS[1]
-    n = 1
+    n = 8
     x = rng.uniform(-1, 1, (n, H, W, C)).astype(np.float32)
     k = (rng.standard_normal((5, 5, C, O)) * 0.02).astype(np.float32)
     dy = rng.uniform(-1, 1, (n, H // 2, W // 2, O)).astype(np.float32)
@@ -117,7 +118,7 @@ def cpu_baseline(batch, budget_s=25.0):
     seconds = sum(work[c] / rates[c] for c in ("fwd", "dx", "dk")) + work["dense"] / rates["fwd"]
     return {"value": 1.0 / seconds, "unit": "iterations/s", "cores": 1, "kind": kind,
             "sample": "reference cpu::conv2d / conv2d_input_grad / conv2d_kernel_grad on layer D1 "
-                      "([1,32,32,64] -> 128, 5x5, s2) once each, one thread; iteration time extrapolated "
+                      "([8,32,32,64] -> 128, 5x5, s2) once each, one thread; iteration time extrapolated "
                       "from the per-class GFLOP/s (%.3f / %.3f / %.3f) over %.0f GFLOP"
                       % (rates["fwd"] / 1e9, rates["dx"] / 1e9, rates["dk"] / 1e9, work["total"] / 1e9),
             "gflops": {c: rates[c] / 1e9 for c in rates}}

@@ -72,7 +72,18 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     if (pair && (!takes_fast_path(veca, vecb) || C % 4 != 0))
         return fail(DH_ENOTSUP, "%s: the paired launch needs dy channels divisible by 16, result channels divisible by 4, 16-byte aligned tensors below 2 GiB", who);
     const int instances = pair ? 2 : 1;
-    const TileCfg cfg = pick_tile(max_m, C);
+    TileCfg cfg = pick_tile(max_m, C);
+    if (takes_fast_path(veca, vecb))
+    {
+        long tiles = 0, slabs = 0;
+        for (int q = 0; q < n_live; ++q)
+        {
+            const long t = (all[q].M + cfg.bm - 1) / cfg.bm * ((C + cfg.bn - 1) / cfg.bn) * instances;
+            tiles += t;
+            slabs += t * ((all[q].K + BK - 1) / BK);
+        }
+        cfg = narrower_if_split(cfg, tiles, slabs);
+    }
     for (int q = 0; q < n_live; ++q)
         total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;
     if (takes_fast_path(veca, vecb))

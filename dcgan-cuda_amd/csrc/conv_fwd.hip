@@ -32,8 +32,13 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     g_operand_bytes = {(size_t)N * H * W * C * 4, (size_t)kh * kw * C * O * 4, C % BK == 0};
     if (pair && !takes_fast_path(veca, vecb))
         return fail(DH_ENOTSUP, "%s: the paired launch needs input channels divisible by 16, output channels divisible by 4, 16-byte aligned tensors below 2 GiB", who);
-    const TileCfg cfg = pick_tile(p.phase[0].M, O);
+    TileCfg cfg = pick_tile(p.phase[0].M, O);
     const int instances = pair ? 2 : 1;
+    if (takes_fast_path(veca, vecb))
+    {
+        const long tiles = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
+        cfg = narrower_if_split(cfg, tiles, tiles * ((p.phase[0].K + BK - 1) / BK));
+    }
     const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
     if (takes_fast_path(veca, vecb))
     {

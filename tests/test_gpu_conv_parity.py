@@ -283,6 +283,45 @@ def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
         be.lib.dh_debug_force_splitk(0)
 
 
+@pytest.mark.parametrize("case", [  # (N, H, W, C, kh, kw, O, stride), operator, tile the launch must take
+    ((64, 64, 64, 16, 3, 3, 128, 2), "fwd", "128x128"),   # 512 square tiles fill the device unsplit
+    ((64, 64, 64, 128, 3, 3, 16, 2), "dx", "128x128"),    # ... the input gradient's four phases
+    ((64, 32, 32, 16, 3, 3, 256, 2), "fwd", "128x64"),    # 256 square tiles: twice as many narrow ones need no split
+    ((64, 8, 8, 64, 5, 5, 256, 2), "fwd", "128x64"),      # a small split launch: narrow tiles, pixels in sorted order
+    ((64, 8, 8, 128, 5, 5, 64, 2), "dx", "128x64"),       # ... input gradient
+    ((64, 8, 8, 64, 5, 5, 256, 2), "dk", "128x128"),      # the filter gradient keeps the square tile
+])
+def test_tile_width_follows_the_size_of_the_launch(be, orc, case):
+    """Forward and input-gradient launches take 128x64 tiles where 128x128 tiles would need a split
+    that the narrower ones avoid or make cheaper; which tile ran is read from the kernel tags of the
+    profiling interface, the result is checked against the oracle."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    if A.device_info()["compute_units"] != 256:
+        pytest.skip("the expected tiles are those of a device with 256 compute units")
+    shape, op, tile = case
+    print("case", case, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(41, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    orc.set_threads(8)
+    A.profile_enable(1)
+    A.profile_reset()
+    try:
+        if op == "fwd":
+            got, exp, scale = be.conv2d(x, k, (s, s)), orc.conv2d(x, k, (s, s)), 1.0
+        elif op == "dx":
+            got, exp, scale = be.conv2d_input_grad(dy, k, s, (H, W)), orc.conv2d_input_grad(dy, k, s, (H, W)), 1.0
+        else:
+            got, exp = be.conv2d_kernel_grad(dy, x, s, pads), orc.conv2d_kernel_grad(dy, x, s, pads)
+            scale = max(1.0, float(np.abs(exp).max()))
+        tags = [r["name"] for r in A.profile_read()]
+    finally:
+        A.profile_enable(0)
+    assert tags == ["conv_igemm_fast<%s,%s>" % (op, tile)], tags
+    close(got, exp, scale=scale, what=op)
+
+
 def test_split_with_more_workgroups_than_the_table_holds(be, orc):
     """40 row tiles cut into 25 splits each are more workgroups than the kernel's workgroup table
     lists (640): the launch falls back to the nested grid in which every tile uses all its splits."""
