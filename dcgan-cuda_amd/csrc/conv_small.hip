@@ -174,11 +174,10 @@ __global__ __launch_bounds__(256) void dx_few_channels(const SmallDxParams p)
 // output pixel m of a 32-pixel tile and loads ITS patch values k = h*40 + j straight from global
 // memory into the register that MFMA number j consumes; the filter (at most 80 x 64 values) is
 // staged in LDS once per workgroup and read from there, one value per lane and MFMA.  A wavefront
-// computes TF_TILES tiles.
+// computes one tile (two, with the second tile's loads in flight during the first's MFMAs, was slower).
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int TF_KH = 40;           // MFMAs per 32-output-channel block; the contraction is padded to 2 * TF_KH
 constexpr int TF_NB = 2;            // 32-channel blocks: up to 64 output channels
-constexpr int TF_TILES = 1;         // 32-pixel tiles per wavefront
 
 struct ThinFwdParams
 {
@@ -198,38 +197,16 @@ struct ThinFwdParams
 __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
 {
     __shared__ float filt[2 * TF_KH * 32 * TF_NB];   // [k][n], zero beyond K and O
-    {
-        // all of a thread's filter loads in flight together (out-of-range elements read element 0 and
-        // are replaced by zero: no branch around a load)
-        constexpr int PER_THREAD = 2 * TF_KH * 32 * TF_NB / 256;
-        float v[PER_THREAD];
-#pragma unroll
-        for (int u = 0; u < PER_THREAD; ++u)
-        {
-            const int e = threadIdx.x + u * 256;
-            const int k = e / (32 * TF_NB), n = e - k * (32 * TF_NB);
-            const bool ok = k < p.K && n < p.O;
-            const float w = p.k[ok ? (size_t)k * p.O + n : 0];
-            v[u] = ok ? w : 0.f;
-        }
-#pragma unroll
-        for (int u = 0; u < PER_THREAD; ++u)
-            filt[threadIdx.x + u * 256] = v[u];
-    }
-    __syncthreads();
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const float* bw = filt + half * TF_KH * (32 * TF_NB) + l32;   // + q * 64 + nb * 32
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
-    const int tiles = (p.pixels + 31) / 32;
-#pragma unroll 1
-    for (int u = 0; u < TF_TILES; ++u)
+    // The wavefront's one tile.  Its patch loads are issued before the filter is staged, so that the
+    // two round trips to memory overlap (a wavefront past the last tile loads nothing: every offset
+    // is out of range).
     {
-        const int tile = (blockIdx.x * 4 + wave) * TF_TILES + u;
-        if (tile >= tiles)
-            break;
+        const int tile = blockIdx.x * 4 + wave;
         const int pix = tile * 32 + l32;
         const bool live = pix < p.pixels;
         uint32_t b, rem, i, j;
@@ -251,6 +228,25 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
             const int off = ok ? base + ((int)di * p.W * p.C + (int)t) * 4 : (int)0x80000000u;
             a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
         }
+        {
+            // all of a thread's filter loads in flight together (out-of-range elements read element 0 and
+            // are replaced by zero: no branch around a load)
+            constexpr int PER_THREAD = 2 * TF_KH * 32 * TF_NB / 256;
+            float v[PER_THREAD];
+#pragma unroll
+            for (int u = 0; u < PER_THREAD; ++u)
+            {
+                const int e = threadIdx.x + u * 256;
+                const int k = e / (32 * TF_NB), n = e - k * (32 * TF_NB);
+                const bool ok = k < p.K && n < p.O;
+                const float w = p.k[ok ? (size_t)k * p.O + n : 0];
+                v[u] = ok ? w : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < PER_THREAD; ++u)
+                filt[threadIdx.x + u * 256] = v[u];
+        }
+        __syncthreads();
         f32x16 acc[TF_NB];
 #pragma unroll
         for (int nb = 0; nb < TF_NB; ++nb)
@@ -517,7 +513,7 @@ int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W,
     p.pixels = N * Ho * Wo;
     p.x_bytes = (uint32_t)x_bytes;
     p.fd_HoWo = FastDiv((uint32_t)Ho * Wo); p.fd_Wo = FastDiv(Wo); p.fd_row = FastDiv(kw * C); p.fd_C = FastDiv(C);
-    const long blocks = ((long)(p.pixels + 31) / 32 + 4 * TF_TILES - 1) / (4 * TF_TILES);
+    const long blocks = ((long)(p.pixels + 31) / 32 + 3) / 4;   // four wavefronts, one 32-pixel tile each
     if (blocks > 0x7fffffffL)
         return 1;
     const int prof = prof_begin("fwd_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
