@@ -16,7 +16,9 @@ Prints ONE JSON line.  Besides the contract fields it carries
 
 `--workload layers` instead sweeps the four DCGAN layer shapes (forward, input gradient, filter
 gradient separately; BASELINE.json config 1) at `--batch`, each timed over a sustained run, and
-prints one JSON line with a row per (layer, operator).
+prints one JSON line with a row per (layer, operator).  `--workload generator --batch 4096` times
+the generator's forward pass alone (BASELINE.json config 4's inference half; config 0 at batch 64).
+`cpu_baseline.mcpu` is the reference's RT_MODE=MCPU runtime (4 workers) on the same sample.
 
 After the timed region a plain device-to-device copy of 256 MiB runs four times: under
 `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its known size calibrates the counters.
@@ -116,7 +118,26 @@ def cpu_baseline(batch, budget_s=25.0):
     rates["dk"] = fl / (time.perf_counter() - t0)
     work = iteration_flops(batch)
     seconds = sum(work[c] / rates[c] for c in ("fwd", "dx", "dk")) + work["dense"] / rates["fwd"]
-    return {"value": 1.0 / seconds, "unit": "iterations/s", "cores": 1, "kind": kind,
+    mcpu = None
+    if kind == "reference":
+        # RT_MODE=MCPU: the same three operators as one node list through the reference's
+        # rt::optimize + ThreadPoolRunner with its 4 workers.  Its optimiser leaves convolution
+        # nodes whole, so what MCPU gains is the overlap of independent nodes (here three; the
+        # iteration's backward pass has two to four per layer).
+        sequential = sum(fl / rates[c] for c in ("fwd", "dx", "dk"))
+        prog = oracle.RefProgram()
+        nodes = [prog.conv2d(x, k, (2, 2), (3, 3))[0], prog.conv2d_input_grad(dy, k, 2, (H, W))[0],
+                 prog.conv2d_kernel_grad(dy, x, 2, (3, 3))[0]]
+        t0 = time.perf_counter()
+        prog.run(nodes, mcpu=True, workers=4)
+        t_mcpu = time.perf_counter() - t0
+        mcpu = {"workers": 4, "sample_seconds": t_mcpu, "sequential_seconds": sequential,
+                "speedup": sequential / t_mcpu, "value": sequential / t_mcpu / seconds,
+                "unit": "iterations/s",
+                "sample": "the same three operators as independent nodes of one list, run by the "
+                          "reference's rt::optimize + cpu::ThreadPoolRunner(4); iteration rate = the "
+                          "one-thread rate x the measured speedup"}
+    return {"value": 1.0 / seconds, "unit": "iterations/s", "cores": 1, "kind": kind, "mcpu": mcpu,
             "sample": "reference cpu::conv2d / conv2d_input_grad / conv2d_kernel_grad on layer D1 "
                       "([8,32,32,64] -> 128, 5x5, s2) once each, one thread; iteration time extrapolated "
                       "from the per-class GFLOP/s (%.3f / %.3f / %.3f) over %.0f GFLOP"
@@ -195,6 +216,66 @@ def layer_sweep(args, A):
     }))
 
 
+def generator_only(args, pkg, A):
+    """BASELINE.json config 4, second half (config 0 at --batch 64): the generator's forward pass
+    alone -- dense 100 -> 4*4*512, four transpose convolutions with bias and relu / tanh in the
+    write-out.  z is resident, the images stay on the device; one step = one pass over the batch."""
+    weights, z, _ = synthetic(args.batch)
+    model = pkg.hostabi.DcganModel(args.batch, seed=1, mode="GPU")
+    model.set_fusion(bool(args.fusion))
+    for name, w in weights.items():
+        model.set_var(name, w)
+    model.set_inputs(z=z)
+    for _ in range(args.warmup):
+        model.generate(to_host=False)
+    model.sync()
+    A.profile_reset()
+    every = max(1, args.profile_every)
+    timer = A.Timer()
+    t0 = time.perf_counter()
+    timer.start()
+    profiled = 0
+    for i in range(args.steps):
+        on = i % every == 0
+        if on:
+            A.profile_enable(1)
+            profiled += 1
+        model.generate(to_host=False)
+        if on:
+            A.profile_enable(0)
+    gpu_ms = timer.stop_ms()
+    model.sync()
+    wall = time.perf_counter() - t0
+    rows = A.profile_read()
+    flops = sum(conv_flops(args.batch, l) for l in LAYERS) + 2.0 * args.batch * 100 * 8192
+    conv_ms = sum(r["ms"] for r in rows)
+    conv_fl = sum(r["flops"] for r in rows)
+    dom = max(rows, key=lambda r: r["ms"])
+    achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "DCGAN generator forward images/sec, fp32", "value": round(args.batch * args.steps / wall, 1),
+        "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[4] (configs[0] at batch 64): DCGAN generator forward only, fp32, batch %d, "
+                               "z dim 100 -> [%d,64,64,3]" % (args.batch, args.batch), "batch": args.batch},
+        "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
+        "step_gflop": round(flops / 1e9, 2), "step_tflops": round(flops / (wall / args.steps) / 1e12, 3),
+        "device": A.device_info(),
+        "roofline": {"kernel": dom["name"], "bound": "mfma", "achieved": round(achieved, 3),
+                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                     "all_conv_kernels": {"tflops": round(conv_fl / (conv_ms * 1e-3) / 1e12, 3),
+                                          "frac": round(conv_fl / (conv_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                                          "ms_per_step": round(conv_ms / max(profiled, 1), 4)},
+                     "kernels": [{"name": r["name"], "launches": r["launches"],
+                                  "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+                                  "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2)}
+                                 for r in sorted(rows, key=lambda r: -r["ms"])]},
+    }))
+    model.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -202,7 +283,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--fusion", type=int, default=1)
-    ap.add_argument("--workload", choices=["iteration", "layers"], default="iteration")
+    ap.add_argument("--workload", choices=["iteration", "layers", "generator"], default="iteration")
     ap.add_argument("--profile-every", type=int, default=5,
                     help="bracket the convolution launches with HIP events in every n-th timed iteration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -214,6 +295,9 @@ def main():
     A = pkg.hipabi
     if args.workload == "layers":
         layer_sweep(args, A)
+        return
+    if args.workload == "generator":
+        generator_only(args, pkg, A)
         return
     weights, z, x = synthetic(args.batch)
     model = pkg.hostabi.DcganModel(args.batch, seed=1, mode="GPU")

@@ -337,7 +337,12 @@ int dg_sync(void)
 
 int dg_generate(void* model, float* images_host)
 {
-    return guarded([&] { ops::Graph::instance().run({M(model).g_out}, {}, {images_host}); });
+    // images_host == nullptr: the images stay on the device and the run is not waited for
+    return guarded([&] {
+        hip::set_sync_each_run(images_host != nullptr);
+        ops::Graph::instance().run({M(model).g_out}, {}, {images_host});
+        hip::set_sync_each_run(true);
+    });
 }
 
 int dg_eval(void* model, const char* what, float* host, long* count)

@@ -144,7 +144,11 @@ class DcganModel:
     def sync(self):
         _check(self.lib.dg_sync())
 
-    def generate(self):
+    def generate(self, to_host=True):
+        """Generator forward pass.  to_host=False leaves the images on the device and does not wait."""
+        if not to_host:
+            _check(self.lib.dg_generate(self.h, None))
+            return None
         out = np.empty((self.batch, 64, 64, 3), np.float32)
         _check(self.lib.dg_generate(self.h, _p(out)))
         return out

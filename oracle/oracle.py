@@ -294,3 +294,75 @@ class XorShift:
     def next_u64(self):
         self.lib.orc_xorshift_next_u64.restype = C.c_uint64
         return int(self.lib.orc_xorshift_next_u64(C.byref(self.state)))
+
+
+class RefProgram:
+    """A node list run by the reference's own runtime (oracle/_ref only): sequentially, as under
+    RT_MODE=CPU (src/cpu/runner.cu:10-14), or by rt::optimize + cpu::ThreadPoolRunner, as under
+    RT_MODE=MCPU (src/ops/graph.cu:180-192; the reference hard-codes 4 workers, :32).  The
+    reference's optimiser does not split convolution nodes (src/runtime/optimizer.cu:239-247,
+    :561-583), so MCPU runs each convolution on one worker and gains only from nodes that are
+    independent of each other."""
+
+    def __init__(self):
+        if not have_ref():
+            raise FileNotFoundError(LIB_REF + " is not built (needs the reference tree)")
+        self.lib = C.CDLL(LIB_REF)
+        self.lib.ref_program_new.restype = C.c_void_p
+        self.p = C.c_void_p(self.lib.ref_program_new())
+        self.keep = []          # operand arrays stay alive as long as the program
+        self.count = 0
+
+    def __del__(self):
+        if getattr(self, "p", None):
+            self.lib.ref_program_free(self.p)
+            self.p = None
+
+    @staticmethod
+    def _ints(v):
+        return (C.c_int * len(v))(*v)
+
+    def _preds(self, preds):
+        return self._ints(list(preds) or [-1]), C.c_int(len(preds))
+
+    def _added(self, idx):
+        self.count += 1
+        assert idx == self.count - 1
+        return idx
+
+    def conv2d(self, x, k, strides, pads, preds=()):
+        x, k = _f32(x), _f32(k)
+        N, H, W, _ = x.shape
+        y = np.zeros((N, -(-H // strides[0]), -(-W // strides[1]), k.shape[3]), np.float32)
+        self.keep += [x, k, y]
+        pa, pn = self._preds(preds)
+        idx = self.lib.ref_node_conv2d(self.p, _p(x), _p(k), _p(y), self._ints(strides),
+                                       C.c_int(pads[0]), C.c_int(pads[1]),
+                                       self._ints(x.shape), self._ints(k.shape), pa, pn)
+        return self._added(idx), y
+
+    def conv2d_input_grad(self, dy, k, stride, in_hw, preds=()):
+        dy, k = _f32(dy), _f32(k)
+        dx = np.zeros((dy.shape[0], in_hw[0], in_hw[1], k.shape[2]), np.float32)
+        self.keep += [dy, k, dx]
+        pa, pn = self._preds(preds)
+        idx = self.lib.ref_node_conv2d_input_grad(self.p, _p(dy), _p(k), _p(dx),
+                                                  self._ints((stride, stride)), self._ints(dy.shape),
+                                                  self._ints(k.shape), self._ints(dx.shape), pa, pn)
+        return self._added(idx), dx
+
+    def conv2d_kernel_grad(self, dy, x, stride, pads, preds=()):
+        dy, x = _f32(dy), _f32(x)
+        kh = x.shape[1] + pads[0] - stride * (dy.shape[1] - 1)
+        kw = x.shape[2] + pads[1] - stride * (dy.shape[2] - 1)
+        dk = np.zeros((kh, kw, x.shape[3], dy.shape[3]), np.float32)
+        self.keep += [dy, x, dk]
+        pa, pn = self._preds(preds)
+        idx = self.lib.ref_node_conv2d_kernel_grad(self.p, _p(dy), _p(x), _p(dk),
+                                                   self._ints((stride, stride)), self._ints(dy.shape),
+                                                   self._ints(x.shape), self._ints(pads), pa, pn)
+        return self._added(idx), dk
+
+    def run(self, outs, mcpu=False, workers=4):
+        self.lib.ref_program_run(self.p, self._ints(outs), C.c_int(len(outs)),
+                                 C.c_int(1 if mcpu else 0), C.c_int(workers))

@@ -107,3 +107,39 @@ def test_generate_and_argmax_bit_exact(cpu_dump):
     clear = (margin[..., -1] - margin[..., -2]) > 1e-5   # exclude numerical ties
     assert np.array_equal(img.argmax(-1)[clear], exp.argmax(-1)[clear])
     assert clear.mean() > 0.95
+
+
+def test_generator_at_batch_4096_is_batch_invariant(cpu_dump):
+    """Generator-only inference at batch 4096 (largest activation [4096,32,32,64], 1.07 GB): too
+    large for the oracle, so the check is a property -- an image does not depend on the batch it
+    is generated in.  The first BATCH latent vectors are the oracle-checked ones; their images
+    must agree with the oracle's to tolerance, and images of repeated latent vectors elsewhere in
+    the batch (its last rows, the rows across the 2 GiB byte offset of the largest activation)
+    must agree with the images of the rows they repeat."""
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    big = 4096
+    w, z, _ = dr.synthetic(BATCH, SEED, pkg.hostabi.var_shapes())
+    rng = np.random.default_rng(5)
+    zb = rng.uniform(-1, 1, (big, 100)).astype(np.float32)
+    zb[:BATCH] = z
+    copies = {big - 1: 17, big - 2: 1000, 2048: 3, 2047: 4000}     # row -> row whose z it repeats
+    for dst, src in copies.items():
+        zb[dst] = zb[src]
+    model = pkg.hostabi.DcganModel(big, SEED, "GPU")
+    try:
+        model.set_fusion(True)
+        for name, val in w.items():
+            model.set_var(name, val)
+        model.set_inputs(z=zb)
+        model.generate(to_host=False)          # device-resident pass, as the benchmark runs it
+        img = model.generate()
+    finally:
+        model.set_fusion(False)
+        model.close()
+    assert np.isfinite(img).all()
+    exp = cpu_dump["g_out"].reshape(BATCH, 64, 64, 3)
+    np.testing.assert_allclose(img[:BATCH], exp, rtol=RTOL, atol=ATOL)
+    for dst, src in copies.items():
+        np.testing.assert_allclose(img[dst], img[src], rtol=RTOL, atol=ATOL)
+    assert len({img[i].tobytes() for i in range(0, big, 97)}) == len(range(0, big, 97))   # rows differ

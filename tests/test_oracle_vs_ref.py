@@ -94,3 +94,21 @@ def test_adam_bit_exact(orc, ref):
     eq(orc.moment_update2(v, g, 0.999, 0.001), ref.moment_update2(v, g, 0.999, 0.001))
     eq(orc.adam_apply(p, m, v, 3e-4, 1e-8), ref.adam_apply(p, m, v, 3e-4, 1e-8))
     eq(orc.vect_update(p, g, -0.1), ref.vect_update(p, g, -0.1))
+
+
+@pytest.mark.parametrize("mcpu", [False, True])
+def test_reference_runtime_runs_the_conv_nodes(ref, mcpu):
+    """The node-list path used for the MCPU baseline timing (the reference's topological sort,
+    rt::optimize and ThreadPoolRunner) gives what the operator functions give."""
+    import oracle
+    N, H, W, C, kh, kw, O, s = 2, 8, 8, 3, 5, 5, 4, 2
+    x, k, dy = rand_conv_inputs(11, N, H, W, C, kh, kw, O, s)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    prog = oracle.RefProgram()
+    a, y = prog.conv2d(x, k, (s, s), pads)
+    b, dx = prog.conv2d_input_grad(dy, k, s, (H, W))
+    c, dk = prog.conv2d_kernel_grad(dy, x, s, pads)
+    prog.run([a, b, c], mcpu=mcpu, workers=4)
+    eq(y, ref.conv2d(x, k, (s, s)))
+    eq(dx, ref.conv2d_input_grad(dy, k, s, (H, W)))
+    eq(dk, ref.conv2d_kernel_grad(dy, x, s, pads))
