@@ -287,6 +287,9 @@ def main():
     ap.add_argument("--profile-every", type=int, default=5,
                     help="bracket the convolution launches with HIP events in every n-th timed iteration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--host-inputs", action="store_true",
+                    help="copy z and the image batch from host memory in every iteration (the PCIe-inclusive "
+                         "rate; the default keeps them resident)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
@@ -307,6 +310,8 @@ def main():
     model.set_inputs(z, x)   # resident from here on
 
     def iteration():
+        if args.host_inputs:
+            model.set_inputs(z, x)   # blocking host-to-device copies, as the reference's Graph::run feeds its inputs
         model.d_step(want_loss=False)
         model.g_step(want_loss=False)
 
@@ -388,7 +393,8 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[3]: full DCGAN training iteration (D step on real+fake, one G step, Adam), "
                                "fp32, batch %d, 64x64x3 images, z dim 100" % args.batch,
-                   "batch": args.batch, "fusion": bool(args.fusion)},
+                   "batch": args.batch, "fusion": bool(args.fusion),
+                   "inputs": "copied from host memory every iteration" if args.host_inputs else "resident in HBM"},
         "gpu_ms_per_step": round(gpu_ms / args.steps, 4),
         "iteration_gflop": round(work["total"] / 1e9, 2),
         "iteration_tflops": round(work["total"] / (wall / args.steps) / 1e12, 3),
