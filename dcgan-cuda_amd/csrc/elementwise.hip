@@ -418,7 +418,11 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     }
     const ColsumCut cut = colsum_cut(rows, cols);
     float* partial = parts_out;
-    if (db && !partial)
+    // one range of rows: its sums are the column sums (the second stage would add zeros to them)
+    const bool single = db && !parts_out && cut.chunks == 1;
+    if (single)
+        partial = db;
+    else if (db && !partial)
     {
         void* ws;
         DH_TRY(workspace(cut.chunks * cols * sizeof(float), &ws, st));
@@ -438,7 +442,7 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     else DH_COLSUM_LAUNCH(colsum_stage1<false>);
 #undef DH_COLSUM_LAUNCH
     DH_LAUNCH_CHECK(who);
-    if (db && !parts_out)
+    if (db && !parts_out && !single)
     {
         hipLaunchKernelGGL(colsum_stage2, dim3((unsigned)((cols + TPB / 64 - 1) / (TPB / 64))), dim3(TPB), 0, st,
                            partial, db, (uint32_t)cols, (uint32_t)cut.chunks);

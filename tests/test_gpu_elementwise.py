@@ -36,7 +36,7 @@ def test_activations_and_grads(be, orc, n):
     np.testing.assert_array_equal(be.add(a, d), orc.add(a, d))
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 3), (4096, 3), (1000, 64), (333, 128), (64, 512), (64, 8192), (5, 300), (4097, 20)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 3), (64, 1), (4096, 3), (1000, 64), (333, 128), (64, 512), (64, 8192), (5, 300), (4097, 20)])
 def test_bias_add_and_grad(be, orc, rows, cols):
     rng = np.random.default_rng(rows * 31 + cols)
     z = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
