@@ -19,6 +19,8 @@ gradient separately; BASELINE.json config 1) at `--batch`, each timed over a sus
 prints one JSON line with a row per (layer, operator).  `--workload generator --batch 4096` times
 the generator's forward pass alone (BASELINE.json config 4's inference half; config 0 at batch 64).
 `cpu_baseline.mcpu` is the reference's RT_MODE=MCPU runtime (4 workers) on the same sample.
+`--workload streaming` times the memory-bound operators (bias, activations, their gradients, Adam)
+on 128 MiB tensors, as algorithmic GB/s against the HBM peak, with a plain copy beside them.
 
 After the timed region a plain device-to-device copy of 256 MiB runs four times: under
 `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its known size calibrates the counters.
@@ -216,6 +218,87 @@ def layer_sweep(args, A):
     }))
 
 
+def streaming_sweep(args, A):
+    """The memory-bound operators of the path (bias add, activations and their gradients, bias
+    gradient, add, the Adam kernels) on tensors of `--elements` floats each (default 2^25 = 128 MiB:
+    the [512,32,32,64] activation of the batch-512 iteration), where the launch itself no longer
+    weighs.  Each operator runs back to back for at least `--sustain-ms` (100 ms; a profiler run
+    wants fewer launches) and at least `--steps` launches between one pair of HIP events;
+    its rate is algorithmic bytes per launch / time per launch against the 8 TB/s HBM peak.  A plain
+    device-to-device copy of the same size (8 B/elem) is timed the same way beside them."""
+    import ctypes as C
+    lib = A.load()
+    n = args.elements
+    cols = 64
+    rows = n // cols
+    n = rows * cols
+    rng = np.random.default_rng(7)
+    host = rng.uniform(-1, 1, n).astype(np.float32)
+    a, b = A.Buf.from_numpy(host), A.Buf.from_numpy(host[::-1].copy())
+    o = A.Buf((n,))
+    m, v = A.Buf.zeros((n,)), A.Buf.zeros((n,))
+    bias = A.Buf.from_numpy(rng.uniform(-1, 1, cols).astype(np.float32))
+    db = A.Buf((cols,))
+    item = A.AdamItem(p=o.ptr, m=m.ptr, v=v.ptr, g1=a.ptr, g2=None, n=n, lrt=1e-4, g1_parts=0, g2_parts=0)
+    items = (A.AdamItem * 1)(item)
+    # name, bytes per element, launch
+    ops = [
+        ("copy (hipMemcpyDtoD)", 8, lambda: lib.dh_memcpy_d2d(o.ptr, a.ptr, n * 4, None)),
+        ("bias_add", 8, lambda: lib.dh_bias_add(a.ptr, bias.ptr, o.ptr, rows, cols, None)),
+        ("relu", 8, lambda: lib.dh_relu(a.ptr, o.ptr, n, None)),
+        ("relu_leaky", 8, lambda: lib.dh_relu_leaky(a.ptr, o.ptr, n, 0.2, None)),
+        ("tanh", 8, lambda: lib.dh_tanh(a.ptr, o.ptr, n, None)),
+        ("sigmoid", 8, lambda: lib.dh_sigmoid(a.ptr, o.ptr, n, None)),
+        ("relu_grad", 12, lambda: lib.dh_relu_grad(a.ptr, b.ptr, o.ptr, n, None)),
+        ("leaky_relu_grad", 12, lambda: lib.dh_leaky_relu_grad(a.ptr, b.ptr, o.ptr, 0.2, n, None)),
+        ("tanh_grad", 12, lambda: lib.dh_tanh_grad(a.ptr, b.ptr, o.ptr, n, None)),
+        ("sigmoid_grad", 12, lambda: lib.dh_sigmoid_grad(a.ptr, b.ptr, o.ptr, n, None)),
+        ("add", 12, lambda: lib.dh_add(a.ptr, b.ptr, o.ptr, n, None)),
+        ("bias_grad", 4, lambda: lib.dh_bias_grad(a.ptr, db.ptr, rows, cols, None)),
+        ("act_bias_grad (leaky)", 12, lambda: lib.dh_act_bias_grad(a.ptr, b.ptr, o.ptr, db.ptr, rows, cols, 2, 0.2, None)),
+        ("moment_update", 12, lambda: lib.dh_moment_update(m.ptr, a.ptr, 0.5, 0.5, n, None)),
+        ("moment_update2", 12, lambda: lib.dh_moment_update2(v.ptr, a.ptr, 0.999, 0.001, n, None)),
+        ("adam_update", 16, lambda: lib.dh_adam_update(o.ptr, m.ptr, v.ptr, 1e-4, 1e-8, n, None)),
+        ("adam_step", 28, lambda: lib.dh_adam_step(o.ptr, m.ptr, v.ptr, a.ptr, 0.5, 0.5, 0.999, 0.001, 1e-4, 1e-8, n, None)),
+        ("adam_step_multi (1 variable)", 28, lambda: lib.dh_adam_step_multi(items, 1, 0.5, 0.5, 0.999, 0.001, 1e-8, None)),
+    ]
+    t = A.Timer()
+    out_rows = []
+    for name, bpe, fn in ops:
+        t.start()
+        for _ in range(3):
+            A.check(fn())
+        est = max(t.stop_ms() / 3, 1e-3)
+        for _ in range(int(0.3 * args.sustain_ms / est) + 1):
+            A.check(fn())
+        A.check(lib.dh_sync())
+        reps = max(args.steps, int(args.sustain_ms / est) + 1)
+        t.start()
+        for _ in range(reps):
+            A.check(fn())
+        ms = t.stop_ms() / reps
+        gbs = bpe * n / (ms * 1e-3) / 1e9
+        out_rows.append({"op": name, "bytes_per_elem": bpe, "launches": reps, "us": round(ms * 1e3, 2),
+                         "gbs": round(gbs, 1), "frac": round(gbs / PEAK_HBM_GBS, 4)})
+    kernels = [r for r in out_rows if not r["op"].startswith("copy")]
+    total_b = sum(r["bytes_per_elem"] * n for r in kernels)
+    total_s = sum(r["us"] * 1e-6 for r in kernels)
+    worst = min(kernels, key=lambda r: r["frac"])
+    print(json.dumps({
+        "metric": "element-wise / bias / Adam kernels: achieved HBM GB/s (algorithmic bytes) against the 8 TB/s peak",
+        "value": round(total_b / total_s / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(total_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "the memory-bound operators of the path on tensors of %d floats (%d x %d for the "
+                               "bias operators); one step = every operator once" % (n, rows, cols), "elements": n},
+        "device": A.device_info(),
+        "roofline": {"kernel": worst["op"], "bound": "hbm", "achieved": worst["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": worst["frac"], "traffic": None,
+                     "note": "the slowest of the operators; every row is in `operators`, the plain copy beside them"},
+        "operators": out_rows,
+    }))
+
+
 def generator_only(args, pkg, A):
     """BASELINE.json config 4, second half (config 0 at --batch 64): the generator's forward pass
     alone -- dense 100 -> 4*4*512, four transpose convolutions with bias and relu / tanh in the
@@ -283,7 +366,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--fusion", type=int, default=1)
-    ap.add_argument("--workload", choices=["iteration", "layers", "generator"], default="iteration")
+    ap.add_argument("--workload", choices=["iteration", "layers", "generator", "streaming"], default="iteration")
+    ap.add_argument("--elements", type=int, default=1 << 25, help="floats per tensor of --workload streaming")
+    ap.add_argument("--sustain-ms", type=float, default=100.0,
+                    help="--workload streaming: time each operator over at least this long a run of launches")
     ap.add_argument("--profile-every", type=int, default=5,
                     help="bracket the convolution launches with HIP events in every n-th timed iteration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -301,6 +387,9 @@ def main():
         return
     if args.workload == "generator":
         generator_only(args, pkg, A)
+        return
+    if args.workload == "streaming":
+        streaming_sweep(args, A)
         return
     weights, z, x = synthetic(args.batch)
     model = pkg.hostabi.DcganModel(args.batch, seed=1, mode="GPU")

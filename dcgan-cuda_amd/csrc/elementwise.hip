@@ -16,11 +16,17 @@ constexpr int TPB = 256;
 
 inline bool aligned16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; }
 
+// Workgroups of a grid-stride kernel over `work` threads' worth of accesses.  Mid-sized launches get
+// 8 workgroups per compute unit and loop; from 8192 workgroups on (8 M floats in 16-byte accesses)
+// every thread makes one access and the loop runs once.  Measured on 16-byte maps: the same speed
+// at 8 M floats, 4-7 % faster without the cap at 16 M, 8 % at 32 M, 20 % at 128 M (the in-place Adam
+// kernels 23-30 %); at 4 M the capped grid is 9 % faster on two-input maps.
 inline unsigned grid_for(size_t work, int per_cu = 8)
 {
     size_t blocks = (work + TPB - 1) / TPB;
     const size_t cap = (size_t)num_cus() * per_cu;
-    if (blocks > cap) blocks = cap;
+    if (blocks > cap && blocks < 8192) blocks = cap;
+    if (blocks > 0x7fffffffu) blocks = 0x7fffffffu;
     return blocks == 0 ? 1u : (unsigned)blocks;
 }
 

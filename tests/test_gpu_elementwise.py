@@ -18,7 +18,9 @@ def close(got, exp, scale=1.0):
     np.testing.assert_allclose(got, exp, rtol=RTOL, atol=ATOL * scale)
 
 
-@pytest.mark.parametrize("n", [1, 3, 255, 1024, 4099, 786432])
+# 8389635 floats: past the size from which the maps run one 16-byte access per thread instead of a
+# capped grid-stride loop (8192 workgroups), with a scalar tail
+@pytest.mark.parametrize("n", [1, 3, 255, 1024, 4099, 786432, 8389635])
 def test_activations_and_grads(be, orc, n):
     rng = np.random.default_rng(n)
     a = rng.uniform(-4, 4, n).astype(np.float32)
@@ -36,7 +38,8 @@ def test_activations_and_grads(be, orc, n):
     np.testing.assert_array_equal(be.add(a, d), orc.add(a, d))
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 3), (64, 1), (4096, 3), (1000, 64), (333, 128), (64, 512), (64, 8192), (5, 300), (4097, 20)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (7, 3), (64, 1), (4096, 3), (1000, 64), (333, 128), (64, 512), (64, 8192), (5, 300), (4097, 20),
+                                       (131073, 64)])
 def test_bias_add_and_grad(be, orc, rows, cols):
     rng = np.random.default_rng(rows * 31 + cols)
     z = rng.uniform(-1, 1, (rows, cols)).astype(np.float32)
@@ -107,7 +110,7 @@ def test_dense(be, orc, m, n, p):
     close(be.mtm_mul(g, w), orc.mtm_mul(g, w))             # g tr(w) : dx
 
 
-@pytest.mark.parametrize("n", [1, 1000, 4099, 3276800])
+@pytest.mark.parametrize("n", [1, 1000, 4099, 3276800, 8389635])
 def test_adam(be, orc, n):
     rng = np.random.default_rng(n)
     p = rng.standard_normal(n).astype(np.float32)
