@@ -14,6 +14,11 @@
  * thread.  The host shim turns non-zero into std::runtime_error, the reference's convention
  * (src/memory/alloc.cu:6-14).
  *
+ * Threads: the reference drives its GPU from one host thread (src/gpu/runner.cu:10-18) and so
+ * does the host mirror here.  Calls from several host threads are allowed when they use
+ * different streams (each stream has a scratch arena of its own) and the same device; calls on
+ * one stream, the dh_profile_* and dh_debug_* hooks, and dh_init must not overlap with other calls.
+ *
  * Each declaration cites the reference interface it stands in for.
  */
 #ifndef DCGAN_HIP_H
