@@ -89,8 +89,7 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     if (takes_fast_path(veca, vecb))
     {
         p.skip = p.posmajor = skipping_pays(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances);
-        order_pixels<MODE_DX>(p, all, n_live, cfg);
-        plan_split<MODE_DX>(p, all, n_live, cfg, pair);
+        plan_launch<MODE_DX>(p, all, n_live, cfg, pair);
     }
     else
         p.splitk = pick_splitk(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances, min_slabs);

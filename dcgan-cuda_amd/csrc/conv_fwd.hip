@@ -43,8 +43,7 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     if (takes_fast_path(veca, vecb))
     {
         p.skip = p.posmajor = skipping_pays(wgs);
-        order_pixels<MODE_FWD>(p, p.phase, 1, cfg);
-        plan_split<MODE_FWD>(p, p.phase, 1, cfg, pair);
+        plan_launch<MODE_FWD>(p, p.phase, 1, cfg, pair);
     }
     else
         p.splitk = pick_splitk(wgs, (p.phase[0].K + BK - 1) / BK);

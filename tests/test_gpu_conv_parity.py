@@ -494,3 +494,41 @@ def test_bad_arguments_are_rejected(be):
         A.check(be.lib.dh_conv2d_fwd(None, x.ptr, x.ptr, 1, 4, 4, 1, 2, 2, 1, 2, 2, 0, 0, 2, 2, None, 0, 0.0, None))
     with pytest.raises(A.HipError):
         A.check(be.lib.dh_conv2d_dk(x.ptr, x.ptr, x.ptr, 0, 4, 4, 1, 2, 2, 1, 2, 2, 2, 2, 0, 0, None))
+
+
+def test_plans_are_kept_per_geometry(be, orc):
+    """The split plan and workgroup table of a launch are remembered per geometry and tuning switches.
+    Launches of two shapes, interleaved and repeated, under changing forced split counts: every
+    result is within tolerance of the oracle, and a repeated launch under the same switches equals
+    its first run to the bit (a plan taken from the wrong entry would give other partial sums, or a
+    table that does not cover the tiles)."""
+    shapes = [(16, 16, 16, 32, 5, 5, 64, 2), (8, 8, 8, 64, 5, 5, 128, 2)]
+    orc.set_threads(8)
+    cases = []
+    for seed, shape in enumerate(shapes):
+        N, H, W, C, kh, kw, O, s = shape
+        x, k, dy = rand_conv_inputs(40 + seed, *shape)
+        pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+        exp = (orc.conv2d(x, k, (s, s)), orc.conv2d_input_grad(dy, k, s, (H, W)), orc.conv2d_kernel_grad(dy, x, s, pads))
+        cases.append((shape, x, k, dy, pads, exp))
+
+    def run(case):
+        (N, H, W, C, kh, kw, O, s), x, k, dy, pads, exp = case
+        got = (be.conv2d(x, k, (s, s)), be.conv2d_input_grad(dy, k, s, (H, W)), be.conv2d_kernel_grad(dy, x, s, pads))
+        for g, e, what in zip(got, exp, ("fwd", "dx", "dk")):
+            close(g, e, scale=max(1.0, float(np.abs(e).max())), what=what)
+        return got
+
+    first = {}
+    try:
+        for splits in (0, 3, 0, 5, 3, 0):
+            be.lib.dh_debug_force_splitk(splits)
+            for ci in (0, 1, 0):
+                got = run(cases[ci])
+                if (splits, ci) in first:
+                    for a, b in zip(first[(splits, ci)], got):
+                        np.testing.assert_array_equal(a, b)
+                else:
+                    first[(splits, ci)] = got
+    finally:
+        be.lib.dh_debug_force_splitk(0)
