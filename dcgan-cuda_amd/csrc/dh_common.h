@@ -19,6 +19,8 @@ int ensure_init();
 // Scratch arena of the current device for launches on `stream`, at least `bytes` large (grows, never
 // shrinks).  Each stream has its own, so that split-K launches on different streams may overlap.
 constexpr int MAX_ARENAS = 8;
+constexpr int STAGE_SLOTS = 16;                       // pinned staging buffers of dh_memcpy_h2d_staged
+constexpr size_t STAGE_MAX_BYTES = size_t(64) << 20;  // larger copies are plain blocking copies
 int workspace(size_t bytes, void** ptr, hipStream_t stream);
 int num_cus();
 

@@ -22,6 +22,11 @@ struct DeviceState
     struct Arena { hipStream_t stream; void* ptr; size_t bytes; };
     Arena arena[MAX_ARENAS] = {};
     int n_arenas = 0;
+    // pinned staging slots of dh_memcpy_h2d_staged, used round-robin; `done` is recorded behind the
+    // slot's copy and waited for before the slot is written again
+    struct Stage { void* host; size_t bytes; hipEvent_t done; bool in_flight; };
+    Stage stage[STAGE_SLOTS] = {};
+    int next_stage = 0;
 };
 
 std::mutex g_mu;
@@ -163,6 +168,44 @@ int dh_memcpy_h2d(void* dst, const void* src, size_t bytes)
     DH_TRY(ensure_init());
     if (bytes == 0) return 0;
     DH_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int dh_memcpy_h2d_staged(void* dst, const void* src, size_t bytes, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(DH_EINVAL, "dh_memcpy_h2d_staged: null pointer");
+    if (bytes > STAGE_MAX_BYTES)
+    {
+        DH_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+        return 0;
+    }
+    std::lock_guard<std::mutex> lock(g_mu);
+    DeviceState& st = g_dev[g_cur];
+    DeviceState::Stage& slot = st.stage[st.next_stage];
+    st.next_stage = (st.next_stage + 1) % STAGE_SLOTS;
+    if (slot.in_flight)
+    {
+        DH_HIP(hipEventSynchronize(slot.done));
+        slot.in_flight = false;
+    }
+    if (!slot.done)
+        DH_HIP(hipEventCreateWithFlags(&slot.done, hipEventDisableTiming));
+    if (bytes > slot.bytes)
+    {
+        if (slot.host)
+            DH_HIP(hipHostFree(slot.host));
+        slot.host = nullptr;
+        slot.bytes = 0;
+        const size_t want = (bytes + 65535) & ~size_t(65535);
+        DH_HIP(hipHostMalloc(&slot.host, want, hipHostMallocDefault));
+        slot.bytes = want;
+    }
+    memcpy(slot.host, src, bytes);
+    DH_HIP(hipMemcpyAsync(dst, slot.host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    DH_HIP(hipEventRecord(slot.done, as_stream(stream)));
+    slot.in_flight = true;
     return 0;
 }
 

@@ -26,6 +26,7 @@ _SIGS = {
     "dh_malloc": [C.POINTER(_vp), _sz],
     "dh_free": [_vp],
     "dh_memcpy_h2d": [_vp, _vp, _sz],
+    "dh_memcpy_h2d_staged": [_vp, _vp, _sz, _vp],
     "dh_memcpy_d2h": [_vp, _vp, _sz],
     "dh_memcpy_d2d": [_vp, _vp, _sz, _vp],
     "dh_memset0": [_vp, _sz, _vp],

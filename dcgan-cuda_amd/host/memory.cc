@@ -65,7 +65,9 @@ void tensor_write(dbl_t* dst_begin, dbl_t* dst_end, const dbl_t* src_host)
 {
     const std::size_t n = dst_end - dst_begin;
     if (program_mode() == ProgramMode::GPU)
-        hip_check(dh_memcpy_h2d(dst_begin, src_host, n * sizeof(dbl_t)), "tensor_write");
+        // stream-ordered behind the work already queued (every instruction runs on the default stream):
+        // the caller's buffer is free on return, and a run that is still executing is not waited for
+        hip_check(dh_memcpy_h2d_staged(dst_begin, src_host, n * sizeof(dbl_t), nullptr), "tensor_write");
     else
         std::copy(src_host, src_host + n, dst_begin);
 }

@@ -54,6 +54,12 @@ int dh_malloc(void** ptr, size_t bytes);
 int dh_free(void* ptr);
 /* tensor_write / tensor_read in GPU mode: src/memory/copy.hxx:29-46 (blocking cudaMemcpy). */
 int dh_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
+/* The same for the inputs a training loop feeds before every run (src/ops/graph.cu:139-147 writes each
+ * fed input with tensor_write): the host buffer is copied into a pinned staging buffer of the library
+ * (16 of them, used in turn) and from there to the device in `stream` order, so src_host may be
+ * reused on return and kernels queued on `stream` afterwards see the data -- but the call does not
+ * wait for the work queued before it, as the blocking copy does.  Copies above 64 MiB are blocking. */
+int dh_memcpy_h2d_staged(void* dst_device, const void* src_host, size_t bytes, void* stream);
 int dh_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
 int dh_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
 /* tensor_fill with zero (src/memory/copy.hxx:7-27) without the host staging buffer. */

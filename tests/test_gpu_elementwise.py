@@ -257,3 +257,32 @@ def test_column_sums_of_unaligned_tensors(be, orc):
     close(db.numpy(), orc.bias_grad(exp), scale=np.sqrt(rows))
     A.check(be.lib.dh_bias_grad(dbuf.ptr + 4, db.ptr, rows, cols, None))
     close(db.numpy(), orc.bias_grad(d2), scale=np.sqrt(rows))
+
+
+def test_staged_host_to_device_copies(be):
+    """dh_memcpy_h2d_staged: the host buffer may be overwritten as soon as the call returns, copies are
+    ordered with the kernels of their stream, and more copies than there are staging buffers (16), of
+    growing and shrinking sizes, all arrive intact."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    lib = be.lib
+    rng = np.random.default_rng(11)
+    sizes = [1, 100, 786432, 6400, 3, 70000, 2, 1 << 20] * 5          # 40 copies
+    host = np.empty(max(sizes), np.float32)
+    bufs, expected = [], []
+    for n in sizes:
+        vals = rng.standard_normal(n).astype(np.float32)
+        host[:n] = vals                                              # the one host buffer, reused every time
+        d = A.Buf((n,))
+        A.check(lib.dh_memcpy_h2d_staged(d.ptr, host.ctypes.data, n * 4, None))
+        host[:n] = -1.0
+        out = A.Buf((n,))
+        A.check(lib.dh_relu(d.ptr, out.ptr, n, None))                # queued behind the copy on the same stream
+        bufs.append((d, out))
+        expected.append(vals)
+    for (d, out), vals in zip(bufs, expected):
+        np.testing.assert_array_equal(d.numpy(), vals)
+        np.testing.assert_array_equal(out.numpy(), np.maximum(vals, 0.0))
+    # nothing to copy / null pointers
+    A.check(lib.dh_memcpy_h2d_staged(bufs[0][0].ptr, host.ctypes.data, 0, None))
+    assert lib.dh_memcpy_h2d_staged(None, host.ctypes.data, 4, None) != 0
