@@ -76,7 +76,10 @@ __global__ __launch_bounds__(256) void dx_few_channels(const SmallDxParams p)
     for (int phase0 = 0; phase0 < nph; phase0 += 4)
     {
         // wave-uniform description of this wavefront's phase (inactive when past the last phase)
-        const int phase = phase0 + wave;
+        // which of the four phases of this round the wavefront takes rotates with the workgroup: the
+        // phases differ in length (9, 6, 6 and 4 taps for 5x5 stride 2) and wavefront w of every workgroup
+        // tends to land on the same SIMD, which would otherwise get all the long ones (measured: 1 %)
+        const int phase = phase0 + ((wave + (int)blockIdx.x) & 3);
         const bool live = phase < nph;
         const int ph = live ? phase / p.sw : 0, pw = live ? phase - (phase / p.sw) * p.sw : 0;
         const int rh = (ph + p.pt) % p.sh, rw = (pw + p.pl) % p.sw;
@@ -176,6 +179,7 @@ __global__ __launch_bounds__(256) void dx_few_channels(const SmallDxParams p)
 // staged in LDS once per workgroup and read from there, one value per lane and MFMA.  A wavefront
 // computes one tile (two, with the second tile's loads in flight during the first's MFMAs, was slower).
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int TF_KH = 40;           // MFMAs per 32-output-channel block; the contraction is padded to 2 * TF_KH
 constexpr int TF_NB = 2;            // 32-channel blocks: up to 64 output channels
 
@@ -194,6 +198,13 @@ struct ThinFwdParams
     FastDiv fd_HoWo, fd_Wo, fd_row, fd_C;
 };
 
+// ROWS: the contraction index is laid out as filter row x 16 (k' = di*16 + dj*C + c; needs kw*C <= 16
+// and kh*16 <= 2*TF_KH), so that a lane's 40 values are ten 16-byte loads of consecutive floats of its
+// input rows instead of forty 4-byte loads -- a quarter of the load instructions for the same lines.
+// Elements of a 16-byte load that belong to no tap (the 16th of a row, columns in the padding) are
+// replaced by zero after the load; the buffer descriptor's range check is per dword, so a load that
+// runs past the end of the tensor still delivers its in-range elements.
+template <bool ROWS>
 __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
 {
     __shared__ float filt[2 * TF_KH * 32 * TF_NB];   // [k][n], zero beyond K and O
@@ -216,17 +227,57 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
         const int base = (((int)b * p.H + h0) * p.W + w0) * p.C * 4;
 
         float a[TF_KH];
-#pragma unroll
-        for (int q = 0; q < TF_KH; ++q)
+        if (ROWS)
         {
-            const int k = half * TF_KH + q;
-            uint32_t di, t, dj, c;
-            p.fd_row.divmod(k, di, t);
-            p.fd_C.divmod(t, dj, c);
-            const bool ok = (int)live & (int)(k < p.K) & (int)((unsigned)(h0 + (int)di) < (unsigned)p.H) &
-                            (int)((unsigned)(w0 + (int)dj) < (unsigned)p.W);
-            const int off = ok ? base + ((int)di * p.W * p.C + (int)t) * 4 : (int)0x80000000u;
-            a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+#pragma unroll
+            for (int u = 0; u < TF_KH / 4; ++u)
+            {
+                const int k0 = half * TF_KH + 4 * u;        // first k' of the chunk
+                const int di = k0 >> 4, t0 = k0 & 15;
+                const bool row_ok = (int)live & (int)(di < p.kh) & (int)((unsigned)(h0 + di) < (unsigned)p.H);
+                const int off = row_ok ? base + (di * p.W * p.C + t0) * 4 : (int)0x80000000u;
+                const f32x4v v = __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(xr, off, 0, 0));
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    const int t = t0 + e;
+                    const int dj = (int)p.fd_C.div((uint32_t)t);
+                    const bool ok = (int)(t < p.row) & (int)((unsigned)(w0 + dj) < (unsigned)p.W);
+                    a[4 * u + e] = ok ? v[e] : 0.f;
+                }
+            }
+            // Pixels of the first image whose patch has padding on its left and holds input row 0: the
+            // 16-byte load of that row would begin before the tensor (a negative offset, which the range
+            // check rejects as a whole, in-range elements included).  Those few pixels take 4-byte loads.
+            if (live && b == 0 && h0 <= 0 && w0 < 0)
+            {
+#pragma unroll
+                for (int q = 0; q < TF_KH; ++q)
+                {
+                    const int kq = half * TF_KH + q;
+                    const int di = kq >> 4, t = kq & 15;
+                    const int dj = (int)p.fd_C.div((uint32_t)t);
+                    const bool ok = (int)(di < p.kh) & (int)(t < p.row) & (int)((unsigned)(h0 + di) < (unsigned)p.H) &
+                                    (int)((unsigned)(w0 + dj) < (unsigned)p.W);
+                    const int off = ok ? base + (di * p.W * p.C + t) * 4 : (int)0x80000000u;
+                    a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+                }
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int q = 0; q < TF_KH; ++q)
+            {
+                const int k = half * TF_KH + q;
+                uint32_t di, t, dj, c;
+                p.fd_row.divmod(k, di, t);
+                p.fd_C.divmod(t, dj, c);
+                const bool ok = (int)live & (int)(k < p.K) & (int)((unsigned)(h0 + (int)di) < (unsigned)p.H) &
+                                (int)((unsigned)(w0 + (int)dj) < (unsigned)p.W);
+                const int off = ok ? base + ((int)di * p.W * p.C + (int)t) * 4 : (int)0x80000000u;
+                a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+            }
         }
         {
             // all of a thread's filter loads in flight together (out-of-range elements read element 0 and
@@ -237,8 +288,16 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
             for (int u = 0; u < PER_THREAD; ++u)
             {
                 const int e = threadIdx.x + u * 256;
-                const int k = e / (32 * TF_NB), n = e - k * (32 * TF_NB);
-                const bool ok = k < p.K && n < p.O;
+                int k = e / (32 * TF_NB);
+                const int n = e - k * (32 * TF_NB);
+                bool ok = k < p.K && n < p.O;
+                if (ROWS)
+                {
+                    // k' = di*16 + t  ->  element (di*row + t) of the filter
+                    const int di = k >> 4, t = k & 15;
+                    ok = di < p.kh && t < p.row && n < p.O;
+                    k = di * p.row + t;
+                }
                 const float w = p.k[ok ? (size_t)k * p.O + n : 0];
                 v[u] = ok ? w : 0.f;
             }
@@ -517,7 +576,10 @@ int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W,
     if (blocks > 0x7fffffffL)
         return 1;
     const int prof = prof_begin("fwd_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
-    hipLaunchKernelGGL(fwd_thin, dim3((unsigned)blocks), dim3(256), 0, st, p);
+    if (kw * C <= 16 && kh * 16 <= 2 * TF_KH)
+        hipLaunchKernelGGL(fwd_thin<true>, dim3((unsigned)blocks), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(fwd_thin<false>, dim3((unsigned)blocks), dim3(256), 0, st, p);
     prof_end(prof, st);
     DH_LAUNCH_CHECK("fwd_thin launch");
     return 0;

@@ -140,6 +140,8 @@ def test_dx_onto_few_channels(be, orc, shape):
     (2, 11, 50, 3, 5, 3, 16, 3),     # stride 3
     (3, 9, 9, 3, 5, 5, 60, 2),       # 60 output channels: the second 32-channel block is partial
     (2, 12, 10, 4, 5, 4, 8, 2),      # contraction of exactly 80
+    (2, 15, 21, 3, 7, 3, 16, 2),     # seven filter rows: the contraction is not laid out by rows (4-byte loads)
+    (2, 12, 14, 4, 4, 5, 24, 1),     # a filter row of 20 values: likewise
 ])
 def test_fwd_from_few_channels(be, orc, shape):
     """Forward convolution from 1-4 input channels with a fused bias + leaky relu and without, against
@@ -160,6 +162,24 @@ def test_fwd_from_few_channels(be, orc, shape):
         close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), exp, what="implicit GEMM")
     finally:
         be.lib.dh_debug_force_generic_conv(0)
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 64, 3, 5, 5, 64, 2), (1, 9, 11, 3, 5, 5, 8, 2), (2, 12, 14, 4, 4, 5, 24, 1)])
+def test_fwd_from_few_channels_reads_only_its_taps(be, orc, shape):
+    """The thin forward kernel loads 16 bytes at a time and discards the elements that belong to no tap
+    (the padding columns, the value after a filter row).  With NaNs planted in the input -- one pixel in
+    the middle, the last pixel of the tensor -- exactly the outputs whose taps cover them may be NaN:
+    the oracle's pattern, element for element."""
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(31, *shape)
+    x[0, H // 2, W // 2, :] = np.nan
+    x[N - 1, H - 1, W - 1, C - 1] = np.nan
+    orc.set_threads(8)
+    exp = orc.conv2d(x, k, (s, s))
+    got = be.conv2d(x, k, (s, s))
+    assert np.isnan(exp).any() and not np.isnan(exp).all()
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(exp))
+    close(got, exp, what="thin forward with NaN inputs")
 
 
 @pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
