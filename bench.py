@@ -47,12 +47,12 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # summaries are kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
     # launch-weighted over the single and the paired instantiation of a tag
-    "conv_igemm_fast<dx,128x64>": 87.1e6,       # 9 single launches of 71.6 MB, 2 paired of 157.0 MB per iteration
-    "conv_igemm_fast<fwd,128x64>": 135.2e6,     # 6 x 119.9 MB, 1 x 226.5 MB
-    "conv_igemm_fast<dk,128x128>": 191.3e6,     # 3 x 126.2 MB, 3 x 256.4 MB
+    "conv_igemm_fast<dx,128x64>": 88.8e6,       # 9 single launches of 73.6 MB, 2 paired of 157.1 MB per iteration
+    "conv_igemm_fast<fwd,128x64>": 135.1e6,     # 6 x 119.9 MB, 1 x 226.3 MB
+    "conv_igemm_fast<dk,128x128>": 191.2e6,     # 3 x 126.1 MB, 3 x 256.2 MB
     "conv_igemm_fast<fwd,128x128>": 182.0e6,    # 2 paired
-    "conv_igemm_fast<dx,128x128>": 172.4e6,     # 1 paired
-    "fwd_thin": 21.7e6,
+    "conv_igemm_fast<dx,128x128>": 171.3e6,     # 1 paired
+    "fwd_thin": 21.8e6,
     "dk_thin": 25.6e6,
     "dx_few_channels": 27.2e6,
 }
