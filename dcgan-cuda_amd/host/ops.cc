@@ -260,7 +260,23 @@ void Graph::run(std::vector<Op*> ops, const std::map<Input*, std::pair<const dbl
         if (outputs[i])
             wanted.push_back(compiled(ops[i]).out_data);
     hip::set_protected_tensors(wanted);
-    rt::execute(list);
+    if (!wanted.empty() && program_mode() == ProgramMode::GPU && hip::sync_each_run())
+    {
+        // the blocking device-to-host copy of the first result waits for the run: no separate wait
+        hip::set_sync_each_run(false);
+        try
+        {
+            rt::execute(list);
+        }
+        catch (...)
+        {
+            hip::set_sync_each_run(true);
+            throw;
+        }
+        hip::set_sync_each_run(true);
+    }
+    else
+        rt::execute(list);
 
     for (std::size_t i = 0; i < outputs.size() && i < ops.size(); ++i)
     {
