@@ -11,11 +11,11 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
     DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     const bool pair = x2 != nullptr || dy2 != nullptr;
     if (!x || !dy || !dk || (pair && (!x2 || !dy2))) return fail(DH_EINVAL, "%s: null tensor", who);
-    if (!pair && !g_force_generic && aligned16(dk))
+    if (!g_force_generic && aligned16(dk))
     {
         float* part = nullptr;
         int splits = 0;
-        const int rc = conv_dk_thin(x, dy, &part, &splits, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left,
+        const int rc = conv_dk_thin(x, dy, x2, dy2, &part, &splits, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left,
                                     as_stream(stream));
         if (rc == 0)
         {
@@ -70,6 +70,16 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
 }  // namespace
 
 extern "C" {
+
+int dh_conv2d_dk_pair_supported(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw)
+{
+    (void)sh;
+    if (ensure_init() != 0) return 0;
+    const double lim = 2147483648.0;
+    if (4.0 * N * H * W * C >= lim || 4.0 * N * Ho * Wo * O >= lim || 4.0 * kh * kw * C * O >= lim) return 0;
+    if (g_force_generic) return 0;
+    return (C % 4 == 0 && O % 4 == 0) || dk_thin_takes(N, H, W, C, Ho, Wo, O, kh, kw, sw) ? 1 : 0;
+}
 
 int dh_conv2d_dk(const float* x, const float* dy, float* dk, int N, int H, int W, int C, int Ho, int Wo,
                  int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left, void* stream)

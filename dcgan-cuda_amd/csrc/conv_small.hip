@@ -370,6 +370,8 @@ struct ThinDkParams
 {
     const float* x;
     const float* dy;
+    const float* x2;      // a second pair of operands, contracted into the same result (images N .. 2N-1), or null
+    const float* dy2;
     float* part;          // [workgroup][M][O]
     int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
     int M;                // kh * kw * C
@@ -452,7 +454,9 @@ __global__ __launch_bounds__(256) void dk_thin(const ThinDkParams p)
         const int j0 = (int)js * DT_SEG;
         const int ih0 = (int)i * p.sh - p.pt;
         const int g0 = (j0 * p.sw - p.pl) * p.C;      // first staged column, in floats from the row start
-        const float* xrow = p.x + ((size_t)b * p.H) * p.W * p.C;
+        const bool second = (int)b >= p.N;       // only with a second pair of operands
+        b -= second ? (uint32_t)p.N : 0u;
+        const float* xrow = (second ? p.x2 : p.x) + ((size_t)b * p.H) * p.W * p.C;
         const ptrdiff_t base = (ptrdiff_t)ih0 * p.W * p.C + g0;
         // every lane loads (from the start of the image where its element does not exist) and the value
         // is dropped afterwards, so that the loads are issued back to back
@@ -465,7 +469,7 @@ __global__ __launch_bounds__(256) void dk_thin(const ThinDkParams p)
             const float v = xrow[ok ? base + r * p.W * p.C + col : 0];
             xv[q] = ok ? v : 0.f;
         }
-        const float* drow = p.dy + (((size_t)b * p.Ho + i) * p.Wo + j0) * p.O;
+        const float* drow = (second ? p.dy2 : p.dy) + (((size_t)b * p.Ho + i) * p.Wo + j0) * p.O;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
         {
@@ -644,22 +648,34 @@ int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int 
 
 // Returns 1 when the shape is not one this kernel takes, 0 after a launch (the caller then adds the
 // *splits slices of M x O partial sums at *part), or an error code.
-int conv_dk_thin(const float* x, const float* dy, float** part, int* splits, int N, int H, int W, int C, int Ho, int Wo,
-                 int O, int kh, int kw, int sh, int sw, int pt, int pl, hipStream_t st)
+// Whether the geometry is one dk_thin takes (the operands must be 16-byte aligned besides).
+bool dk_thin_takes(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sw)
+{
+    const int M = kh * kw * C, row = kw * C;
+    const int rsw = (DT_SEG - 1) * sw * C + row;
+    const int rs = rsw + ((row - rsw) % 32 + 32) % 32;
+    return !(M > DT_MT * 32 || O > DT_OMAX || O % 4 != 0 || kh * rs > DT_XMAX || kh * rsw > 64 * DT_XPL ||
+             (long)N * Ho * Wo < 2048 || (double)N * H * W * C >= 2147483647.0);
+}
+
+// x2 / dy2: a second pair of operands whose filter gradient is added to the first's (both null: one pair).
+int conv_dk_thin(const float* x, const float* dy, const float* x2, const float* dy2, float** part, int* splits, int N,
+                 int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pt, int pl, hipStream_t st)
 {
     const int M = kh * kw * C, row = kw * C;
     const int rsw = (DT_SEG - 1) * sw * C + row;
     const int rs = rsw + ((row - rsw) % 32 + 32) % 32;   // rs = row (mod 32): the 32 lanes of a fragment read hit 32 banks
-    if (M > DT_MT * 32 || O > DT_OMAX || O % 4 != 0 || kh * rs > DT_XMAX || kh * rsw > 64 * DT_XPL ||
-        (reinterpret_cast<uintptr_t>(dy) & 15) != 0 || (long)N * Ho * Wo < 2048 || (double)N * H * W * C >= 2147483647.0)
+    const int images = x2 ? 2 * N : N;
+    if (!dk_thin_takes(N, H, W, C, Ho, Wo, O, kh, kw, sw) || (reinterpret_cast<uintptr_t>(dy) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(dy2) & 15) != 0)
         return 1;
     ThinDkParams p{};
-    p.x = x; p.dy = dy;
+    p.x = x; p.dy = dy; p.x2 = x2; p.dy2 = dy2;
     p.N = N; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.O = O; p.kh = kh; p.kw = kw;
     p.sh = sh; p.sw = sw; p.pt = pt; p.pl = pl;
     p.M = M; p.row = row; p.rsw = rsw; p.rs = rs;
     p.segs_per_row = (Wo + DT_SEG - 1) / DT_SEG;
-    const long total = (long)N * Ho * p.segs_per_row;
+    const long total = (long)images * Ho * p.segs_per_row;
     if (total > 0x7fffffffL)
         return 1;
     p.total_segs = (int)total;
@@ -675,7 +691,7 @@ int conv_dk_thin(const float* x, const float* dy, float** part, int* splits, int
     void* ws;
     DH_TRY(workspace((size_t)wgs * M * O * sizeof(float), &ws, st));
     p.part = static_cast<float*>(ws);
-    const int prof = prof_begin("dk_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
+    const int prof = prof_begin("dk_thin", 2.0 * images * Ho * Wo * O * kh * kw * C, st);
     hipLaunchKernelGGL(dk_thin, dim3((unsigned)wgs), dim3(256), 0, st, p);
     prof_end(prof, st);
     DH_LAUNCH_CHECK("dk_thin launch");

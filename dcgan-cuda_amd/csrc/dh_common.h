@@ -57,8 +57,11 @@ int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W,
 // Filter gradient of a thin input (at most 96 filter elements per output channel, at most 64 output
 // channels): writes *splits slices of partial sums to the scratch arena and returns them in *part for
 // the caller to add up; same return convention.
-int conv_dk_thin(const float* x, const float* dy, float** part, int* splits, int N, int H, int W, int C, int Ho, int Wo,
-                 int O, int kh, int kw, int sh, int sw, int pt, int pl, hipStream_t st);
+// x2 / dy2 (both null, or both set): a second pair of operands contracted into the same result.
+int conv_dk_thin(const float* x, const float* dy, const float* x2, const float* dy2, float** part, int* splits, int N,
+                 int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pt, int pl, hipStream_t st);
+// Whether conv_dk_thin takes this geometry (16-byte aligned operands assumed).
+bool dk_thin_takes(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sw);
 
 // Test and tuning switches (dh_debug_force_generic_conv, dh_debug_force_splitk).
 extern bool g_force_generic;  // route every convolution through the general kernel

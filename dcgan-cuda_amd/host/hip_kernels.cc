@@ -474,8 +474,13 @@ bool pairable(const ConvCall& c)
     const double k_bytes = 4.0 * g.kh * g.kw * g.C * g.O, lim = 2147483648.0;
     // the paired launches need the buffer-load kernel, whose k-slabs of 16 must not straddle filter taps
     const bool tapwise = c.kind == 0 ? g.C % 16 == 0 : c.kind == 1 ? g.O % 16 == 0 : true;
-    return tapwise && g.C % 4 == 0 && g.O % 4 == 0 && in_bytes < lim && out_bytes < lim && k_bytes < lim && aligned(c.a) &&
-           aligned(c.b) && aligned(c.out) && aligned(c.bias);
+    const bool sizes_ok = in_bytes < lim && out_bytes < lim && k_bytes < lim && aligned(c.a) && aligned(c.b) &&
+                          aligned(c.out) && aligned(c.bias);
+    // the filter gradient of a thin input (the image layer) has a paired kernel of its own
+    if (c.kind == 2 && sizes_ok &&
+        dh_conv2d_dk_pair_supported(g.N, g.H, g.W, g.C, g.Ho, g.Wo, g.O, g.kh, g.kw, g.sh, g.sw) == 1)
+        return true;
+    return tapwise && g.C % 4 == 0 && g.O % 4 == 0 && sizes_ok;
 }
 
 bool same_call(const ConvCall& x, const ConvCall& y)

@@ -153,7 +153,10 @@ int dh_conv2d_dk(const float* x, const float* dy, float* dk,
  * They need the buffer-load kernel (channel counts divisible by 4 and, for the channels the product
  * contracts over -- the input's for fwd, dy's for dx -- by 16; 16-byte aligned tensors below 2 GiB)
  * and return DH_ENOTSUP otherwise; results agree with the single calls to rounding
- * (the contraction may be split differently). */
+ * (the contraction may be split differently).  dh_conv2d_dk_pair also takes the thin-input filter
+ * gradient (at most 96 filter elements per output channel, at most 64 output channels: the image
+ * layer); dh_conv2d_dk_pair_supported tells a caller that plans its launches ahead whether a geometry
+ * is one the paired filter gradient takes (1) or not (0), 16-byte aligned tensors assumed. */
 int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
                        int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left, int Ho, int Wo,
                        const float* bias, int act, float alpha, void* stream);
@@ -163,6 +166,7 @@ int dh_conv2d_dx_pair(const float* dy1, const float* dy2, const float* k, float*
 int dh_conv2d_dk_pair(const float* x1, const float* dy1, const float* x2, const float* dy2, float* dk, int N, int H,
                       int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left,
                       void* stream);
+int dh_conv2d_dk_pair_supported(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw);
 
 /* ---- bias and activations: coalesced, vectorised, one pass over HBM ----------------------------- */
 

@@ -552,3 +552,23 @@ def test_plans_are_kept_per_geometry(be, orc):
                     first[(splits, ci)] = got
     finally:
         be.lib.dh_debug_force_splitk(0)
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 64, 3, 5, 5, 64, 2), (4, 70, 37, 2, 3, 3, 48, 2), (8, 36, 36, 3, 5, 5, 60, 2)])
+def test_paired_filter_gradient_of_a_thin_input(be, orc, shape):
+    """dk(x1, dy1) + dk(x2, dy2) of the image layer as one launch of the thin-input kernel (the second
+    pair of operands are images N .. 2N-1 of its contraction), against the sum of the oracle's two
+    gradients; the capability query says so beforehand, and says no for a shape the kernel refuses."""
+    N, H, W, C, kh, kw, O, s = shape
+    x1, k, dy1 = rand_conv_inputs(51, *shape)
+    x2, _, dy2 = rand_conv_inputs(52, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    Ho, Wo = dy1.shape[1:3]
+    assert be.lib.dh_conv2d_dk_pair_supported(N, H, W, C, Ho, Wo, O, kh, kw, s, s) == 1
+    assert be.lib.dh_conv2d_dk_pair_supported(2, 8, 8, 3, 4, 4, 6, 5, 5, 2, 2) == 0
+    orc.set_threads(8)
+    exp = orc.conv2d_kernel_grad(dy1, x1, s, pads).astype(np.float64) + orc.conv2d_kernel_grad(dy2, x2, s, pads)
+    got = be.conv2d_kernel_grad_pair(dy1, x1, dy2, x2, s, pads)
+    close(got, exp.astype(np.float32), scale=max(1.0, float(np.abs(exp).max())), what="paired thin filter gradient")
+    again = be.conv2d_kernel_grad_pair(dy1, x1, dy2, x2, s, pads)
+    np.testing.assert_array_equal(got, again)

@@ -47,8 +47,9 @@ def gpu_dump(fusion):
 
 
 def test_paired_plan_is_shorter():
-    """With pairing the discriminator step issues nine launches fewer: layers 1-3 forward, input
-    gradient and filter gradient of the two towers each become one launch."""
+    """With pairing the discriminator step issues ten launches fewer: layers 1-3 forward, input
+    gradient and filter gradient of the two towers each become one launch, and so does the image
+    layer's filter gradient."""
     import __graft_entry__ as ge
     pkg = ge.load_package()
     counts = {}
@@ -67,7 +68,7 @@ def test_paired_plan_is_shorter():
             model.set_fusion(False)
             model.set_pairing(True)
             model.close()
-    assert counts[False] - counts[True] == 9, counts
+    assert counts[False] - counts[True] == 10, counts
 
 
 @pytest.mark.parametrize("fusion", [False, True, "unpaired"])
