@@ -53,7 +53,7 @@ MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FET
     "conv_igemm_fast<fwd,128x128>": 182.0e6,    # 2 paired
     "conv_igemm_fast<dx,128x128>": 171.3e6,     # 1 paired
     "fwd_thin": 21.8e6,
-    "dk_thin": 25.6e6,
+    "dk_thin": 35.8e6,     # launch-weighted: one paired launch (both towers) and one single per iteration
     "dx_few_channels": 27.2e6,
 }
 
