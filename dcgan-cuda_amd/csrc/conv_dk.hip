@@ -50,6 +50,7 @@ int conv_dk(const char* who, const float* x, const float* dy, const float* x2, c
     if (takes_fast_path(veca, vecb))
     {
         p.skip = N % BK == 0;
+        g_prof_issued = 0.0;
         plan_launch<MODE_DK>(p, p.phase, 1, cfg, pair);
     }
     else

@@ -89,6 +89,7 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     if (takes_fast_path(veca, vecb))
     {
         p.skip = p.posmajor = skipping_pays(total_tiles_m * ((C + cfg.bn - 1) / cfg.bn) * instances);
+        g_prof_issued = 0.0;
         plan_launch<MODE_DX>(p, all, n_live, cfg, pair);
     }
     else
@@ -102,6 +103,7 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     // one launch covers up to MAX_PHASES phases; the operator's FLOPs are split evenly over launches
     const int launches = (n_live + MAX_PHASES - 1) / MAX_PHASES > 0 ? (n_live + MAX_PHASES - 1) / MAX_PHASES : 1;
     g_prof_flops = 2.0 * N * Ho * Wo * O * kh * kw * C * instances / launches;
+    g_prof_issued /= launches;
     for (int z0 = 0; z0 < n_live; z0 += MAX_PHASES)
     {
         const int nz = n_live - z0 < MAX_PHASES ? n_live - z0 : MAX_PHASES;

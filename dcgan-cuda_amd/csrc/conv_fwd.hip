@@ -43,6 +43,7 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     if (takes_fast_path(veca, vecb))
     {
         p.skip = p.posmajor = skipping_pays(wgs);
+        g_prof_issued = 0.0;
         plan_launch<MODE_FWD>(p, p.phase, 1, cfg, pair);
     }
     else

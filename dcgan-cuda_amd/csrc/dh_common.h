@@ -30,7 +30,8 @@ int num_cus();
 // Level 1 times the convolution kernels only (a few dozen launches per training iteration, so the
 // events barely disturb it); level 2 also times the reductions, dense and element-wise kernels.
 bool profiling(int level = 1);
-int prof_begin(const char* name, double work, hipStream_t st, int level = 1);
+// `issued` (convolution kernels): the FLOPs the matrix cores are issued for the launch, 0 = not known.
+int prof_begin(const char* name, double work, hipStream_t st, int level = 1, double issued = 0.0);
 void prof_end(int handle, hipStream_t st);
 // Brackets the launches of one scope.  Memory-bound kernels report algorithmic BYTES as their work
 // and carry the prefix "hbm:" in their name.

@@ -16,13 +16,13 @@ struct ProfRecord
 {
     hipEvent_t e0, e1;
     int tag;
-    double work;
+    double work, issued;
 };
 struct ProfTotal
 {
     char name[96];
     long launches;
-    double ms, work;
+    double ms, work, issued;
 };
 int g_level = 0;   // 0 off, 1 convolution kernels, 2 every tagged kernel
 std::vector<ProfRecord> g_open;      // begun, not yet ended
@@ -57,13 +57,14 @@ hipEvent_t take_event()
 
 bool profiling(int level) { return g_level >= level; }
 
-int prof_begin(const char* name, double work, hipStream_t st, int level)
+int prof_begin(const char* name, double work, hipStream_t st, int level, double issued)
 {
     if (g_level < level)
         return -1;
     ProfRecord r{};
     r.tag = tag_of(name);
     r.work = work;
+    r.issued = issued;
     r.e0 = take_event();
     r.e1 = take_event();
     (void)hipEventRecord(r.e0, st);
@@ -120,6 +121,7 @@ int dh_profile_read(char* buf, size_t buf_len)
         t.launches += 1;
         t.ms += ms;
         t.work += r.work;
+        t.issued += r.issued;
         g_pool.push_back(r.e0);
         g_pool.push_back(r.e1);
     }
@@ -131,7 +133,7 @@ int dh_profile_read(char* buf, size_t buf_len)
     {
         if (!buf || used >= buf_len)
             break;
-        const int w = snprintf(buf + used, buf_len - used, "%s\t%ld\t%.6f\t%.0f\n", t.name, t.launches, t.ms, t.work);
+        const int w = snprintf(buf + used, buf_len - used, "%s\t%ld\t%.6f\t%.0f\t%.0f\n", t.name, t.launches, t.ms, t.work, t.issued);
         if (w < 0 || (size_t)w >= buf_len - used)
             return fail(DH_EINVAL, "dh_profile_read: buffer too small");
         used += (size_t)w;

@@ -178,6 +178,9 @@ int dh_memcpy_h2d_staged(void* dst, const void* src, size_t bytes, void* stream)
     if (!dst || !src) return fail(DH_EINVAL, "dh_memcpy_h2d_staged: null pointer");
     if (bytes > STAGE_MAX_BYTES)
     {
+        // too large to stage: a blocking copy, ordered behind what `stream` holds by waiting for it
+        // (streams made by dh_stream_create do not synchronise with the null stream by themselves)
+        DH_HIP(hipStreamSynchronize(as_stream(stream)));
         DH_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
         return 0;
     }
@@ -243,7 +246,24 @@ int dh_stream_create(void** stream)
 
 int dh_stream_destroy(void* stream)
 {
-    DH_HIP(hipStreamDestroy(as_stream(stream)));
+    DH_TRY(ensure_init());
+    hipStream_t s = as_stream(stream);
+    DH_HIP(hipStreamSynchronize(s));
+    {
+        // the stream's scratch arena goes with it (the table holds at most MAX_ARENAS streams)
+        std::lock_guard<std::mutex> lock(g_mu);
+        DeviceState& st = g_dev[g_cur];
+        for (int i = 0; i < st.n_arenas; ++i)
+            if (st.arena[i].stream == s && s != nullptr)
+            {
+                if (st.arena[i].ptr)
+                    DH_HIP(hipFree(st.arena[i].ptr));
+                st.arena[i] = st.arena[st.n_arenas - 1];
+                st.arena[--st.n_arenas] = DeviceState::Arena{nullptr, nullptr, 0};
+                break;
+            }
+    }
+    DH_HIP(hipStreamDestroy(s));
     return 0;
 }
 

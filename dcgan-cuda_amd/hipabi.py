@@ -40,6 +40,11 @@ _SIGS = {
     "dh_event_record": [_vp, _vp],
     "dh_event_elapsed_ms": [_vp, _vp, C.POINTER(_f)],
     "dh_workspace_reserve": [_sz],
+    "dh_pool_alloc": [C.POINTER(_vp), _sz],
+    "dh_pool_free": [_vp],
+    "dh_pool_reserve": [_sz],
+    "dh_pool_trim": [],
+    "dh_pool_stats": [C.POINTER(_sz)] * 4,
     "dh_debug_force_generic_conv": [_i],
     "dh_debug_force_splitk": [_i],
     "dh_profile_enable": [_i],
@@ -166,6 +171,13 @@ class Buf:
             pass
 
 
+def pool_stats():
+    """hipMalloc calls, bytes held, bytes handed out and their peak of the tensor pool (dh_pool_*)."""
+    v = [_sz() for _ in range(4)]
+    check(load().dh_pool_stats(*[C.byref(x) for x in v]))
+    return dict(zip(("hipmallocs", "held", "in_use", "peak"), (x.value for x in v)))
+
+
 def device_info():
     name = C.create_string_buffer(256)
     cus, khz, mem = _i(), _i(), _sz()
@@ -209,14 +221,15 @@ def profile_reset():
 
 
 def profile_read():
-    """[{name, launches, ms, flops}] per kernel tag since the last reset.  `flops` is the algorithmic
-    work of the launches: FLOPs, or bytes for the tags that start with "hbm:"."""
+    """[{name, launches, ms, flops, issued}] per kernel tag since the last reset.  `flops` is the
+    algorithmic work of the launches: FLOPs, or bytes for the tags that start with "hbm:"; `issued` the
+    FLOPs the matrix cores were issued (0.0 where the launch site does not account for them)."""
     buf = C.create_string_buffer(1 << 16)
     check(load().dh_profile_read(buf, len(buf)))
     rows = []
     for line in buf.value.decode().splitlines():
-        name, n, ms, fl = line.split("\t")
-        rows.append({"name": name, "launches": int(n), "ms": float(ms), "flops": float(fl)})
+        name, n, ms, fl, issued = line.split("\t")
+        rows.append({"name": name, "launches": int(n), "ms": float(ms), "flops": float(fl), "issued": float(issued)})
     return rows
 
 

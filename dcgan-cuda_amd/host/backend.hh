@@ -8,18 +8,14 @@
 // -- there is no silent CPU fallback.
 #pragma once
 
+#include "hip_table.hh"
 #include "mode.hh"
 #include "rt_graph.hh"
-
-using kernel_f = void (*)(rt::Node*);
 
 namespace hip
 {
 
-// Indexed by rt::Node::type.  Entries 20 and 31 are nullptr exactly as in the reference
-// (conv2d_bias_add lowers to mat_rvect_add, its gradient to mat_sum_cols); the softmax family
-// (4, 5, 6, 18) is not on the convolution path and is nullptr as well.
-extern kernel_f kernels_list[512];
+// kernels_list[512] and the plain table runner are declared in hip_table.hh.
 
 // Issues every instruction of the list on the backend's stream, in order, WITHOUT a device
 // synchronisation between instructions; returns after one synchronisation at the end.
@@ -53,6 +49,12 @@ void forget_plans();
 // blocking copy or hip::synchronize() waits for them).  On by default.
 void set_sync_each_run(bool on);
 bool sync_each_run();
+
+// Copies `count` values from host memory into the device tensor at `dst` for the runs that follow: on a
+// copy stream of the backend's own, behind the work queued so far; the launch stream waits for the copy
+// in front of the first step that touches the tensor (or at the end of the next run).  src_host may be
+// reused on return.
+void feed(dbl_t* dst, const dbl_t* src_host, std::size_t count);
 
 void* stream();  // hipStream_t the backend launches on
 void synchronize();

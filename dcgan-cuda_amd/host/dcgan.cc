@@ -1,6 +1,8 @@
 #include "dcgan.hh"
 #include "images.hh"
+#include "npz.hh"
 
+#include <cstddef>
 #include <cstring>
 #include <stdexcept>
 
@@ -356,10 +358,46 @@ int dg_eval(void* model, const char* what, float* host, long* count)
     });
 }
 
+int dg_eval_many(void* model, const char* names, float** hosts, int count)
+{
+    return guarded([&] {
+        std::vector<ops::Op*> targets;
+        std::vector<dbl_t*> outs;
+        const std::string all(names);
+        std::size_t at = 0;
+        while (at <= all.size() && (int)targets.size() < count)
+        {
+            std::size_t end = all.find(';', at);
+            if (end == std::string::npos)
+                end = all.size();
+            targets.push_back(lookup(M(model), all.substr(at, end - at)));
+            outs.push_back(hosts[targets.size() - 1]);
+            at = end + 1;
+        }
+        if ((int)targets.size() != count)
+            throw std::runtime_error("dg_eval_many: fewer names than count");
+        ops::Graph::instance().run(targets, {}, outs);
+    });
+}
+
 int dg_save_vars(void*, const char* path) { return guarded([&] { ops::Graph::instance().save_vars(path); }); }
 int dg_load_vars(void*, const char* path) { return guarded([&] { ops::Graph::instance().load_vars(path); }); }
 int dg_save_state(void*, const char* path) { return guarded([&] { ops::Graph::instance().save_state(path); }); }
 int dg_load_state(void*, const char* path) { return guarded([&] { ops::Graph::instance().load_state(path); }); }
+
+int dg_npz_inspect(const char* path, long* arrays, long* elements)
+{
+    return guarded([&] {
+        const std::vector<npz::Array> all = npz::load(path);
+        long n = 0;
+        for (const npz::Array& a : all)
+            n += (long)a.data.size();
+        if (arrays)
+            *arrays = (long)all.size();
+        if (elements)
+            *elements = n;
+    });
+}
 
 int dg_images_normalize(const unsigned char* pix, long count, float* out)
 {
@@ -378,6 +416,27 @@ int dg_images_save_samples(const float* data, long width, long height, const cha
 {
     return guarded([&] { images::save_samples(data, (std::size_t)width, (std::size_t)height, path); });
 }
+
+// sizeof(rt::Node) followed by the offset of every field a kernel-table entry reads, in declaration
+// order: type, in1, in2, in3, out1, out2, cons1..4, len1..3, intconst, intconst2, sizes1..3,
+// int_cons1, int_cons2, alpha_leaky.  Returns the number of values written (at most n).
+#pragma GCC diagnostic push
+#pragma GCC diagnostic ignored "-Winvalid-offsetof"
+int dg_node_layout(unsigned long* out, int n)
+{
+    using N = rt::Node;
+    const unsigned long v[] = {sizeof(N), offsetof(N, type), offsetof(N, in1), offsetof(N, in2), offsetof(N, in3),
+                               offsetof(N, out1), offsetof(N, out2), offsetof(N, cons1), offsetof(N, cons2),
+                               offsetof(N, cons3), offsetof(N, cons4), offsetof(N, len1), offsetof(N, len2),
+                               offsetof(N, len3), offsetof(N, intconst), offsetof(N, intconst2), offsetof(N, sizes1),
+                               offsetof(N, sizes2), offsetof(N, sizes3), offsetof(N, int_cons1), offsetof(N, int_cons2),
+                               offsetof(N, alpha_leaky)};
+    const int count = (int)(sizeof(v) / sizeof(v[0]));
+    for (int i = 0; i < count && i < n; ++i)
+        out[i] = v[i];
+    return count < n ? count : n;
+}
+#pragma GCC diagnostic pop
 
 int dg_last_launch_count(void*) { return hip::last_launch_count(); }
 

@@ -69,6 +69,9 @@ int dg_generate(void* model, float* images_host);
 //   "grad:g_loss:<var index>", "grad:d_loss:<var index>", "grad:g_loss:x_fake" (d g_loss / d g_out)
 // Returns the number of elements through *count; host may be NULL to query the size only.
 int dg_eval(void* model, const char* what, float* host, long* count);
+// The same for `count` tensors named in one ';'-separated string, evaluated in ONE run of the graph
+// (shared upstream tensors are computed once); hosts[i] receives the i-th tensor.
+int dg_eval_many(void* model, const char* names, float** hosts, int count);
 // Trainable variables to / from a file (numpy .npz when the path ends in ".npz"); the whole training
 // state (all variables, Adam moments and step counters) as .npz.  The model argument is unused: the
 // operator graph is a process-wide singleton.
@@ -76,11 +79,17 @@ int dg_save_vars(void* model, const char* path);
 int dg_load_vars(void* model, const char* path);
 int dg_save_state(void* model, const char* path);
 int dg_load_state(void* model, const char* path);
+// Reads a .npz archive with the reader behind dg_load_vars / dg_load_state and reports how many arrays
+// and elements it holds; fails (with the reader's message) on anything it would refuse to load.
+int dg_npz_inspect(const char* path, long* arrays, long* elements);
 // Image helpers (host/images.hh): 8-bit pixels to [-1, 1]; images <dir>/<6-digit index>.ppm for
 // idx_beg <= index < idx_end as one normalised batch; width x height generated images as one PPM mosaic.
 int dg_images_normalize(const unsigned char* pix, long count, float* out);
 int dg_images_load(const char* dir, long idx_beg, long idx_end, float* out);
 int dg_images_save_samples(const float* data, long width, long height, const char* path);
+// Layout of this library's rt::Node (size, then field offsets): equal to the reference's record
+// (src/runtime/node.hh:215-242) field for field, which a test checks against a build of the reference.
+int dg_node_layout(unsigned long* out, int n);
 // Number of rt::Node instructions / fused launches of the last run.
 int dg_last_schedule_size(void* model);
 int dg_last_launch_count(void* model);

@@ -1,7 +1,6 @@
-// The HIP backend seen from the operator graph: a kernel table indexed by rt::Node::type and a
-// runner, i.e. the drop-in for gpu::kernels_list / gpu::run (src/gpu/kernels.cu:23-61,
-// src/gpu/runner.cu:10-18).  Each table entry decodes the node exactly as the reference's GPU
-// entry does (citations per function) and makes one C-ABI call; nothing else happens here.
+// The HIP backend's planning runner: the instruction list of a run is pattern-matched into fused and
+// paired C-ABI calls (or issued node by node through the kernel table of hip_table.cc when fusion is
+// off), without the reference's per-node device synchronisation (src/gpu/runner.cu:10-18).
 #include "backend.hh"
 
 #include <algorithm>
@@ -24,104 +23,13 @@ namespace hip
 namespace
 {
 
-void* g_stream = nullptr;  // the default stream; every launch of the backend is ordered on it
 int g_fusion = -1;         // -1: not decided yet (reads DCGAN_HIP_FUSE)
 int g_last_launches = 0;    // steps of the plan that ran last
 bool g_pairing = true;     // issue same-filter convolutions of independent towers as one launch (part of fusion)
 
 #define CK(call) hip_check((call), #call)
 
-struct ConvGeom
-{
-    int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
-};
-
-// conv2d forward.  Node fields: src/runtime/node.cu:118-141; decode: src/gpu/conv2d.cu:13-40.
-ConvGeom geom_conv2d(const rt::Node* n)
-{
-    ConvGeom g;
-    g.N = n->sizes1[0]; g.H = n->sizes1[1]; g.W = n->sizes1[2]; g.C = n->sizes1[3];
-    g.kh = n->sizes2[0]; g.kw = n->sizes2[1]; g.O = n->sizes2[3];
-    g.sh = n->intconst[0]; g.sw = n->intconst[1];
-    const int pad_h = n->int_cons1, pad_w = n->int_cons2;  // totals; the part before is half, rounded down
-    g.pt = pad_h / 2; g.pl = pad_w / 2;
-    g.Ho = (g.H + pad_h - g.kh) / g.sh + 1;
-    g.Wo = (g.W + pad_w - g.kw) / g.sw + 1;
-    return g;
-}
-
-// conv2d input gradient.  Fields: src/runtime/node.cu:171-193; decode: src/gpu/conv2d.cu:70-98
-// (one stride for both axes, pads re-derived from the extents).
-ConvGeom geom_input_grad(const rt::Node* n)
-{
-    ConvGeom g;
-    g.N = n->sizes1[0]; g.Ho = n->sizes1[1]; g.Wo = n->sizes1[2]; g.O = n->sizes1[3];
-    g.kh = n->sizes2[0]; g.kw = n->sizes2[1]; g.C = n->sizes2[2];
-    g.sh = g.sw = n->intconst[0];
-    g.H = n->intconst2[0]; g.W = n->intconst2[1];
-    g.pt = ((g.Ho - 1) * g.sh - g.H + g.kh) / 2;
-    g.pl = ((g.Wo - 1) * g.sw - g.W + g.kw) / 2;
-    return g;
-}
-
-// conv2d filter gradient.  Fields: src/runtime/node.cu:195-217; decode: src/gpu/conv2d.cu:119-146
-// (filter extent derived as H + pad - s*(Ho-1)).
-ConvGeom geom_kernel_grad(const rt::Node* n)
-{
-    ConvGeom g;
-    g.N = n->sizes2[0]; g.H = n->sizes2[1]; g.W = n->sizes2[2]; g.C = n->sizes2[3];
-    g.Ho = n->sizes1[1]; g.Wo = n->sizes1[2]; g.O = n->sizes1[3];
-    g.sh = n->intconst[0]; g.sw = n->intconst[1];
-    const int pad_h = n->intconst2[0], pad_w = n->intconst2[1];
-    g.pt = pad_h / 2; g.pl = pad_w / 2;
-    g.kh = g.H + pad_h - g.sh * (g.Ho - 1);
-    g.kw = g.W + pad_w - g.sw * (g.Wo - 1);
-    return g;
-}
-
-// conv2d_transpose forward = input gradient of the conv whose "y" is this op's input.
-// Fields: src/runtime/node.cu:219-243; decode: src/gpu/conv2d.cu:167-196.
-ConvGeom geom_transpose(const rt::Node* n)
-{
-    ConvGeom g;
-    g.N = n->sizes2[0]; g.Ho = n->sizes2[1]; g.Wo = n->sizes2[2]; g.O = n->sizes2[3];
-    g.kh = n->sizes3[0]; g.kw = n->sizes3[1]; g.C = n->sizes3[2];
-    g.sh = n->intconst[0]; g.sw = n->intconst[1];
-    g.H = n->sizes1[1]; g.W = n->sizes1[2];
-    g.pt = ((g.Ho - 1) * g.sh - g.H + g.kh) / 2;
-    g.pl = ((g.Wo - 1) * g.sw - g.W + g.kw) / 2;
-    return g;
-}
-
-// conv2d_transpose input gradient = forward conv of dy.  Fields: src/runtime/node.cu:245-267;
-// decode: src/gpu/conv2d.cu:214-241.
-ConvGeom geom_transpose_input_grad(const rt::Node* n)
-{
-    ConvGeom g;
-    g.N = n->sizes1[0]; g.H = n->sizes1[1]; g.W = n->sizes1[2]; g.C = n->sizes2[2];
-    g.kh = n->sizes2[0]; g.kw = n->sizes2[1]; g.O = n->sizes2[3];
-    g.sh = g.sw = n->intconst[0];
-    g.Ho = n->intconst2[0]; g.Wo = n->intconst2[1];
-    g.pt = ((g.Ho - 1) * g.sh + g.kh - g.H) / 2;
-    g.pl = ((g.Wo - 1) * g.sw + g.kw - g.W) / 2;
-    return g;
-}
-
-// conv2d_transpose filter gradient = conv2d filter gradient with dy in the role of the image and
-// the transpose's input in the role of the output gradient.  Fields: src/runtime/node.cu:269-294;
-// decode: src/gpu/conv2d.cu:264-289.
-ConvGeom geom_transpose_kernel_grad(const rt::Node* n)
-{
-    ConvGeom g;
-    g.N = n->sizes2[0]; g.Ho = n->sizes2[1]; g.Wo = n->sizes2[2]; g.O = n->sizes2[3];  // transpose input
-    g.H = n->sizes1[1]; g.W = n->sizes1[2]; g.C = n->sizes1[3];                        // dy
-    g.kh = n->sizes3[0]; g.kw = n->sizes3[1];
-    g.sh = n->intconst[0]; g.sw = n->intconst[1];
-    g.pt = ((g.Ho - 1) * g.sh + g.kh - g.H) / 2;
-    g.pl = ((g.Wo - 1) * g.sw + g.kw - g.W) / 2;
-    return g;
-}
-
+// conv_fwd / conv_dx: one C-ABI call for a decoded geometry (with optional epilogue)
 void conv_fwd(const ConvGeom& g, const dbl_t* x, const dbl_t* k, dbl_t* y, const dbl_t* bias, int act, float alpha)
 {
     CK(dh_conv2d_fwd(x, k, y, g.N, g.H, g.W, g.C, g.kh, g.kw, g.O, g.sh, g.sw, g.pt, g.pl, g.Ho, g.Wo, bias, act,
@@ -134,70 +42,7 @@ void conv_dx(const ConvGeom& g, const dbl_t* dy, const dbl_t* k, dbl_t* dx, cons
                     alpha, g_stream));
 }
 
-void conv_dk(const ConvGeom& g, const dbl_t* x, const dbl_t* dy, dbl_t* dk)
-{
-    CK(dh_conv2d_dk(x, dy, dk, g.N, g.H, g.W, g.C, g.Ho, g.Wo, g.O, g.kh, g.kw, g.sh, g.sw, g.pt, g.pl, g_stream));
-}
 
-// ---- table entries -----------------------------------------------------------------------------
-void k_conv2d(rt::Node* n) { conv_fwd(geom_conv2d(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f); }
-void k_conv2d_input_grad(rt::Node* n) { conv_dx(geom_input_grad(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f); }
-void k_conv2d_kernel_grad(rt::Node* n) { conv_dk(geom_kernel_grad(n), n->in2, n->in1, n->out1); }
-void k_conv2d_transpose(rt::Node* n) { conv_dx(geom_transpose(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f); }
-void k_conv2d_transpose_input_grad(rt::Node* n)
-{
-    conv_fwd(geom_transpose_input_grad(n), n->in1, n->in2, n->out1, nullptr, DH_ACT_NONE, 0.f);
-}
-void k_conv2d_transpose_kernel_grad(rt::Node* n) { conv_dk(geom_transpose_kernel_grad(n), n->in1, n->in2, n->out1); }
-
-// src/gpu/matmul.cu:88-150 (matmul, mvrow_add, matmul_add, tmat_mat_mul, mat_tmat_mul hosts)
-void k_mat_mat_mul(rt::Node* n) { CK(dh_gemm_nn(n->in1, n->in2, nullptr, n->out1, n->len1, n->len2, n->len3, g_stream)); }
-void k_mat_rvect_add(rt::Node* n) { CK(dh_bias_add(n->in1, n->in2, n->out1, n->len1, n->len2, g_stream)); }
-void k_mat_mul_add(rt::Node* n) { CK(dh_gemm_nn(n->in1, n->in2, n->in3, n->out1, n->len1, n->len2, n->len3, g_stream)); }
-void k_tmat_mat_mul(rt::Node* n) { CK(dh_gemm_tn(n->in1, n->in2, n->out1, n->len1, n->len2, n->len3, g_stream)); }
-void k_mat_tmat_mul(rt::Node* n) { CK(dh_gemm_nt(n->in1, n->in2, n->out1, n->len1, n->len2, n->len3, g_stream)); }
-// src/gpu/sum.cu:216-243
-void k_mat_sum_rows(rt::Node* n) { CK(dh_mat_sum_rows(n->in1, n->out1, n->len1, n->len2, g_stream)); }
-void k_mat_sum_cols(rt::Node* n) { CK(dh_bias_grad(n->in1, n->out1, n->len1, n->len2, g_stream)); }
-void k_mse(rt::Node* n) { CK(dh_mse(n->in1, n->in2, n->out1, n->len1, n->len2, g_stream)); }
-void k_mse_grad(rt::Node* n) { CK(dh_mse_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
-void k_argmax_acc(rt::Node* n) { CK(dh_argmax_acc(n->in1, n->in2, n->out1, n->len1, n->len2, g_stream)); }
-void k_add(rt::Node* n) { CK(dh_add(n->in1, n->in2, n->out1, n->len1, g_stream)); }
-// src/gpu/relu.cu:68-104
-void k_relu(rt::Node* n) { CK(dh_relu(n->in1, n->out1, n->len1, g_stream)); }
-void k_relu_leaky(rt::Node* n) { CK(dh_relu_leaky(n->in1, n->out1, n->len1, n->alpha_leaky, g_stream)); }
-void k_relu_grad(rt::Node* n) { CK(dh_relu_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
-void k_leaky_relu_grad(rt::Node* n) { CK(dh_leaky_relu_grad(n->in1, n->in2, n->out1, n->cons1, n->len1, g_stream)); }
-// src/gpu/sigmoid.cu:124-180
-void k_sigmoid(rt::Node* n) { CK(dh_sigmoid(n->in1, n->out1, n->len1, g_stream)); }
-void k_tanh(rt::Node* n) { CK(dh_tanh(n->in1, n->out1, n->len1, g_stream)); }
-void k_sigmoid_grad(rt::Node* n) { CK(dh_sigmoid_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
-void k_tanh_grad(rt::Node* n) { CK(dh_tanh_grad(n->in1, n->in2, n->out1, n->len1, g_stream)); }
-void k_sigmoid_cross_entropy(rt::Node* n) { CK(dh_sigmoid_cross_entropy(n->in1, n->in2, n->out1, n->len1, g_stream)); }
-void k_sigmoid_cross_entropy_grad(rt::Node* n)
-{
-    CK(dh_sigmoid_cross_entropy_grad(n->in1, n->in2, n->out1, n->len1, g_stream));
-}
-// src/gpu/update.cu:56-96
-void k_update(rt::Node* n) { CK(dh_sgd_update(n->out1, n->in1, n->in2, n->len1, g_stream)); }
-void k_moment_update(rt::Node* n) { CK(dh_moment_update(n->out1, n->in1, n->cons1, n->cons2, n->len1, g_stream)); }
-void k_moment_update2(rt::Node* n) { CK(dh_moment_update2(n->out1, n->in1, n->cons1, n->cons2, n->len1, g_stream)); }
-
-// The step counter lives on the host (node->out2) and is advanced at issue time; the corrected
-// rate is formed in float exactly as src/gpu/update.cu:81-93 does.
-float adam_advance(rt::Node* n)
-{
-    dbl_t* t = n->out2;
-    const dbl_t lr = n->cons1, beta1 = n->cons2, beta2 = n->cons3;
-    ++*t;
-    return lr * std::sqrt(1 - std::pow(beta2, *t)) / (1 - std::pow(beta1, *t));
-}
-
-void k_adam_update(rt::Node* n)
-{
-    const float lrt = adam_advance(n);
-    CK(dh_adam_update(n->out1, n->in1, n->in2, lrt, n->cons4, n->len1, g_stream));
-}
 
 // ---- fusion plan -------------------------------------------------------------------------------
 // A step is either one node run through the table or one fused call standing for several nodes.
@@ -343,9 +188,9 @@ dbl_t* parts_buffer(const dbl_t* grad, std::size_t floats)
     if (slot.second < floats)
     {
         if (slot.first)
-            CK(dh_free(slot.first));
+            CK(dh_pool_free(slot.first));
         void* q = nullptr;
-        CK(dh_malloc(&q, floats * sizeof(dbl_t)));
+        CK(dh_pool_alloc(&q, floats * sizeof(dbl_t)));
         slot = {static_cast<dbl_t*>(q), floats};
     }
     return slot.first;
@@ -1023,46 +868,6 @@ std::unordered_set<const dbl_t*> g_keep;
 
 }  // namespace
 
-kernel_f kernels_list[512] = {
-    k_mat_mat_mul,                   // 0
-    k_mat_rvect_add,                 // 1
-    k_sigmoid,                       // 2
-    k_mse,                           // 3
-    nullptr,                         // 4  softmax                (not on the convolution path)
-    nullptr,                         // 5  log_softmax            (")
-    nullptr,                         // 6  softmax_cross_entropy  (")
-    k_conv2d,                        // 7
-    k_relu,                          // 8
-    k_relu_leaky,                    // 9
-    k_tanh,                          // 10
-    k_mse_grad,                      // 11
-    k_sigmoid_grad,                  // 12
-    k_mat_mul_add,                   // 13
-    k_tmat_mat_mul,                  // 14
-    k_mat_tmat_mul,                  // 15
-    k_mat_sum_rows,                  // 16
-    k_mat_sum_cols,                  // 17
-    nullptr,                         // 18 softmax_cross_entropy_grad (")
-    k_relu_grad,                     // 19
-    nullptr,                         // 20 conv2d_bias_add: lowered to mat_rvect_add by the operator
-    k_update,                        // 21
-    k_sigmoid_cross_entropy,         // 22
-    k_sigmoid_cross_entropy_grad,    // 23
-    k_conv2d_input_grad,             // 24
-    k_conv2d_kernel_grad,            // 25
-    k_argmax_acc,                    // 26
-    k_moment_update,                 // 27
-    k_moment_update2,                // 28
-    k_adam_update,                   // 29
-    k_leaky_relu_grad,               // 30
-    nullptr,                         // 31 conv2d_bias_add_grad: lowered to mat_sum_cols
-    k_tanh_grad,                     // 32
-    k_conv2d_transpose,              // 33
-    k_conv2d_transpose_input_grad,   // 34
-    k_conv2d_transpose_kernel_grad,  // 35
-    k_add,                           // 36
-};
-
 void set_fusion(bool on)
 {
     g_fusion = on ? 1 : 0;
@@ -1087,14 +892,104 @@ namespace { bool g_sync_each_run = true; }
 void set_sync_each_run(bool on) { g_sync_each_run = on; }
 bool sync_each_run() { return g_sync_each_run; }
 
-void* stream() { return g_stream; }
+void* stream() { return g_stream; }   // hip_table.hh: the default stream
 
-void synchronize() { CK(dh_stream_sync(g_stream)); }
+namespace { void wait_for_feeds(const Step* s); }
+
+void synchronize()
+{
+    wait_for_feeds(nullptr);
+    CK(dh_stream_sync(g_stream));
+}
 
 void set_protected_tensors(const std::vector<const dbl_t*>& tensors)
 {
     g_keep.clear();
     g_keep.insert(tensors.begin(), tensors.end());
+}
+
+// ---- inputs fed from host memory --------------------------------------------------------------
+// The reference copies every fed input with a blocking cudaMemcpy in front of the run
+// (src/ops/graph.cu:139-147), which first drains whatever is still executing.  Here the copy goes to a
+// stream of its own: it starts once the work queued so far has finished (an earlier run may still read
+// the tensor), and the launch stream waits for it only in front of the first step that touches the
+// tensor -- the image batch of a discriminator step arrives while the generator's forward pass runs.
+namespace
+{
+struct Feed { const dbl_t* begin; const dbl_t* end; void* done; };
+std::vector<Feed> g_feeds;             // copies the launch stream has not been ordered behind yet
+void* g_copy_stream = nullptr;
+constexpr int FEED_EVENTS = 32;        // ring of (queued-so-far, copy-done) event pairs
+void* g_feed_events[FEED_EVENTS] = {};
+int g_next_feed_event = 0;
+
+void* next_feed_event()
+{
+    void*& e = g_feed_events[g_next_feed_event];
+    g_next_feed_event = (g_next_feed_event + 1) % FEED_EVENTS;
+    if (!e)
+        CK(dh_event_create(&e));
+    return e;
+}
+
+bool node_touches(const rt::Node* n, const Feed& f)
+{
+    if (!n)
+        return false;
+    for (const dbl_t* t : {n->in1, n->in2, n->in3, (const dbl_t*)n->out1})
+        if (t >= f.begin && t < f.end)
+            return true;
+    return false;
+}
+
+bool step_touches(const Step& s, const Feed& f)
+{
+    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+        if (node_touches(n, f))
+            return true;
+    if (s.act_ref >= f.begin && s.act_ref < f.end)
+        return true;
+    for (const Step& g : s.group)
+        if (step_touches(g, f))
+            return true;
+    return false;
+}
+
+// Orders the launch stream behind every outstanding copy (all == true) or behind those `s` touches.
+void wait_for_feeds(const Step* s)
+{
+    for (std::size_t i = 0; i < g_feeds.size();)
+        if (!s || step_touches(*s, g_feeds[i]))
+        {
+            CK(dh_stream_wait_event(g_stream, g_feeds[i].done));
+            g_feeds.erase(g_feeds.begin() + (long)i);
+        }
+        else
+            ++i;
+}
+}  // namespace
+
+void feed(dbl_t* dst, const dbl_t* src_host, std::size_t count)
+{
+    if (count == 0)
+        return;
+    if (!g_copy_stream)
+        CK(dh_stream_create(&g_copy_stream));
+    // an outstanding copy into the same tensor is ordered before this one by the copy stream itself
+    for (std::size_t i = 0; i < g_feeds.size();)
+        if (g_feeds[i].begin < dst + count && dst < g_feeds[i].end)
+            g_feeds.erase(g_feeds.begin() + (long)i);
+        else
+            ++i;
+    void* queued = next_feed_event();
+    void* done = next_feed_event();
+    CK(dh_event_record(queued, g_stream));
+    CK(dh_stream_wait_event(g_copy_stream, queued));
+    CK(dh_memcpy_h2d_staged(dst, src_host, count * sizeof(dbl_t), g_copy_stream));
+    CK(dh_event_record(done, g_copy_stream));
+    g_feeds.push_back(Feed{dst, dst + count, done});
+    if (g_feeds.size() > FEED_EVENTS / 4)   // far more inputs than a graph feeds: do not outrun the event ring
+        wait_for_feeds(nullptr);
 }
 
 void run_async(rt::NodesList& tasks)
@@ -1105,7 +1000,13 @@ void run_async(rt::NodesList& tasks)
     if (it == g_plans.end())
         it = g_plans.emplace(key, make_plan(tasks.nodes(), g_keep, key.fuse)).first;
     for (const Step& s : it->second.steps)
+    {
+        if (!g_feeds.empty())
+            wait_for_feeds(&s);
         issue(s);
+    }
+    // whatever the run did not touch: results are read back with copies that only see the launch stream
+    wait_for_feeds(nullptr);
     g_last_launches = (int)it->second.steps.size();
 }
 
@@ -1120,6 +1021,12 @@ void run(rt::NodesList& tasks)
 void forget_plans()
 {
     g_plans.clear();
+    // the row-range-sum buffers belong to the plans that named them; blocks go back to the pool, which
+    // hands them out again in stream order (see dh_pool_free), so no wait is needed here
+    for (auto& kv : g_parts_pool)
+        if (kv.second.first)
+            CK(dh_pool_free(kv.second.first));
+    g_parts_pool.clear();
 }
 
 }  // namespace hip

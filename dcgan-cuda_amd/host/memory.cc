@@ -47,7 +47,7 @@ dbl_t* tensor_alloc(std::size_t size)
     if (program_mode() == ProgramMode::GPU)
     {
         void* p = nullptr;
-        hip_check(dh_malloc(&p, size * sizeof(dbl_t)), "tensor_alloc");
+        hip_check(dh_pool_alloc(&p, size * sizeof(dbl_t)), "tensor_alloc");
         return static_cast<dbl_t*>(p);
     }
     return new dbl_t[size];
@@ -56,7 +56,7 @@ dbl_t* tensor_alloc(std::size_t size)
 void tensor_free(dbl_t* ptr)
 {
     if (program_mode() == ProgramMode::GPU)
-        hip_check(dh_free(ptr), "tensor_free");
+        hip_check(dh_pool_free(ptr), "tensor_free");
     else
         delete[] ptr;
 }

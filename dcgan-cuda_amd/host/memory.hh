@@ -1,6 +1,6 @@
 // Tensor storage behind the operator graph (reference: src/memory/alloc.hh:9-14,
-// src/memory/copy.hh:8-18).  In GPU mode the calls go through the C ABI (dh_malloc, dh_free,
-// dh_memcpy_*, dh_memset0) and a failing HIP call surfaces as std::runtime_error, the reference's
+// src/memory/copy.hh:8-18).  In GPU mode the calls go through the C ABI (dh_pool_alloc, dh_pool_free:
+// blocks of a pooled allocator, so lowering operators again makes no hipMalloc; dh_memcpy_*, dh_memset0) and a failing HIP call surfaces as std::runtime_error, the reference's
 // convention (src/memory/alloc.cu:6-14); in the CPU modes tensors are plain host arrays.
 #pragma once
 

@@ -147,6 +147,8 @@ std::vector<Array> load(const std::string& path)
     const std::uint32_t cd_off = get32(&buf[(std::size_t)eocd + 16]);
     if (count == 0xffff || cd_off == 0xffffffffu)
         bad(path, "zip64 archives are not supported");
+    if ((std::uint64_t)cd_off + cd_size > (std::uint64_t)file_size)
+        bad(path, "central directory lies outside the file");
     std::vector<unsigned char> cd(cd_size);
     std::fseek(f, (long)cd_off, SEEK_SET);
     if (std::fread(cd.data(), 1, cd.size(), f) != cd.size())
@@ -161,19 +163,27 @@ std::vector<Array> load(const std::string& path)
         const std::uint32_t csize = get32(&cd[at + 20]), usize = get32(&cd[at + 24]);
         const std::uint16_t nlen = get16(&cd[at + 28]), xlen = get16(&cd[at + 30]), clen = get16(&cd[at + 32]);
         const std::uint32_t local_off = get32(&cd[at + 42]);
+        if (at + 46 + (std::size_t)nlen + xlen + clen > cd.size())
+            bad(path, "corrupt central directory (entry runs past its end)");
         std::string member(reinterpret_cast<const char*>(&cd[at + 46]), nlen);
-        at += 46 + nlen + xlen + clen;
+        at += 46 + (std::size_t)nlen + xlen + clen;
         if (method != 0)
             bad(path, "member '" + member + "' is compressed; write the file with numpy.savez, not savez_compressed");
         if (csize == 0xffffffffu || usize == 0xffffffffu || local_off == 0xffffffffu)
             bad(path, "member '" + member + "' needs zip64, which is not supported");
+        if (csize != usize)
+            bad(path, "member '" + member + "': stored and original sizes differ");
         unsigned char lh[30];
+        if ((std::uint64_t)local_off + 30 > (std::uint64_t)file_size)
+            bad(path, "member '" + member + "' lies outside the file");
         std::fseek(f, (long)local_off, SEEK_SET);
         if (std::fread(lh, 1, 30, f) != 30 || get32(lh) != 0x04034b50)
             bad(path, "corrupt local header of '" + member + "'");
-        const long data_off = (long)local_off + 30 + get16(lh + 26) + get16(lh + 28);
+        const std::uint64_t data_off = (std::uint64_t)local_off + 30 + get16(lh + 26) + get16(lh + 28);
+        if (data_off + usize > (std::uint64_t)file_size)
+            bad(path, "truncated member '" + member + "'");
         std::vector<unsigned char> raw(usize);
-        std::fseek(f, data_off, SEEK_SET);
+        std::fseek(f, (long)data_off, SEEK_SET);
         if (std::fread(raw.data(), 1, raw.size(), f) != raw.size())
             bad(path, "truncated member '" + member + "'");
         // .npy: magic, version, header length (2 bytes for v1, 4 for v2/3), python dict literal
@@ -190,28 +200,53 @@ std::vector<Array> load(const std::string& path)
             const std::size_t k = dict.find("'" + key + "'");
             if (k == std::string::npos)
                 bad(path, "'" + member + "': no " + key + " in the .npy header");
-            return dict.find(':', k) + 1;
+            const std::size_t colon = dict.find(':', k);
+            if (colon == std::string::npos)
+                bad(path, "'" + member + "': malformed " + key + " in the .npy header");
+            return colon + 1;
         };
-        std::size_t d0 = dict.find('\'', value_after("descr"));
-        const std::string descr = dict.substr(d0 + 1, dict.find('\'', d0 + 1) - d0 - 1);
+        const std::size_t d0 = dict.find('\'', value_after("descr"));
+        const std::size_t d1 = d0 == std::string::npos ? d0 : dict.find('\'', d0 + 1);
+        if (d1 == std::string::npos)
+            bad(path, "'" + member + "': malformed descr in the .npy header");
+        const std::string descr = dict.substr(d0 + 1, d1 - d0 - 1);
         if (descr != "<f4" && descr != "<f8")
             bad(path, "'" + member + "' has dtype " + descr + "; float32 or float64 expected");
-        if (dict.compare(dict.find_first_not_of(' ', value_after("fortran_order")), 5, "False") != 0)
+        const std::size_t fo = dict.find_first_not_of(' ', value_after("fortran_order"));
+        if (fo == std::string::npos || dict.compare(fo, 5, "False") != 0)
             bad(path, "'" + member + "' is in Fortran order");
         Array a;
         a.name = member.size() > 4 && member.compare(member.size() - 4, 4, ".npy") == 0
                      ? member.substr(0, member.size() - 4) : member;
-        std::size_t s0 = dict.find('(', value_after("shape")), s1 = dict.find(')', s0);
-        std::size_t num = 0;
+        const std::size_t s0 = dict.find('(', value_after("shape"));
+        const std::size_t s1 = s0 == std::string::npos ? s0 : dict.find(')', s0);
+        if (s1 == std::string::npos)
+            bad(path, "'" + member + "': no shape tuple in the .npy header");
+        const std::size_t esz = descr == "<f4" ? 4 : 8, payload = raw.size() - hstart - hlen;
+        std::size_t num = 0, n = 1;
         bool in_num = false;
         for (std::size_t i = s0 + 1; i <= s1; ++i)
         {
             const char c = dict[i];
-            if (c >= '0' && c <= '9') { num = num * 10 + (std::size_t)(c - '0'); in_num = true; }
-            else if (in_num) { a.shape.push_back(num); num = 0; in_num = false; }
+            if (c >= '0' && c <= '9')
+            {
+                if (num > payload)   // no dimension can exceed the payload: stops the digits from wrapping
+                    bad(path, "'" + member + "': data size does not match its shape");
+                num = num * 10 + (std::size_t)(c - '0');
+                in_num = true;
+            }
+            else if (in_num)
+            {
+                // the element count stays within the payload, so neither it nor n * esz can wrap
+                if (num != 0 && n > payload / num)
+                    bad(path, "'" + member + "': data size does not match its shape");
+                n *= num;
+                a.shape.push_back(num);
+                num = 0;
+                in_num = false;
+            }
         }
-        const std::size_t n = a.size(), esz = descr == "<f4" ? 4 : 8;
-        if (hstart + hlen + n * esz != raw.size())
+        if (n > payload / esz || n * esz != payload)
             bad(path, "'" + member + "': data size does not match its shape");
         a.data.resize(n);
         const unsigned char* src = &raw[hstart + hlen];

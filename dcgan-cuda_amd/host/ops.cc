@@ -238,7 +238,10 @@ void Graph::run(std::vector<Op*> ops, const std::map<Input*, std::pair<const dbl
     {
         compile_(kv.first);
         dbl_t* dst = compiled(kv.first).out_data;
-        tensor_write(dst, dst + kv.second.second.total(), kv.second.first);
+        if (program_mode() == ProgramMode::GPU)
+            hip::feed(dst, kv.second.first, (std::size_t)kv.second.second.total());
+        else
+            tensor_write(dst, dst + kv.second.second.total(), kv.second.first);
     }
 
     // the execution order depends only on the requested operators: computed once, then reused

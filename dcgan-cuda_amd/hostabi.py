@@ -42,10 +42,12 @@ def load():
         lib.dg_g_step.argtypes = [C.c_void_p, _fp]
         lib.dg_generate.argtypes = [C.c_void_p, _fp]
         lib.dg_eval.argtypes = [C.c_void_p, C.c_char_p, _fp, C.POINTER(C.c_long)]
+        lib.dg_eval_many.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(_fp), C.c_int]
         lib.dg_last_schedule_size.argtypes = [C.c_void_p]
         lib.dg_last_launch_count.argtypes = [C.c_void_p]
         for name in ("dg_save_vars", "dg_load_vars", "dg_save_state", "dg_load_state"):
             getattr(lib, name).argtypes = [C.c_void_p, C.c_char_p]
+        lib.dg_npz_inspect.argtypes = [C.c_char_p, C.POINTER(C.c_long), C.POINTER(C.c_long)]
         lib.dg_images_normalize.argtypes = [C.c_char_p, C.c_long, _fp]
         lib.dg_images_load.argtypes = [C.c_char_p, C.c_long, C.c_long, _fp]
         lib.dg_images_save_samples.argtypes = [_fp, C.c_long, C.c_long, C.c_char_p]
@@ -93,7 +95,9 @@ class DcganModel:
             if cpu_backend is None:
                 raise HostError("a CPU mode needs a backend library (the host library holds the HIP backend only)")
             self._backend = C.CDLL(cpu_backend, mode=C.RTLD_GLOBAL)
-            self._backend.orc_register_backend()
+            # a library named *_f64.so registers the float64-accumulating flavour of the oracle
+            reg = "orc_register_backend_f64" if cpu_backend.endswith("_f64.so") else "orc_register_backend"
+            getattr(self._backend, reg)()
         self.batch = batch
         self.h = self.lib.dg_create(batch, seed)
         if not self.h:
@@ -160,6 +164,21 @@ class DcganModel:
         _check(self.lib.dg_eval(self.h, what.encode(), _p(out), None))
         return out.reshape(shape) if shape is not None else out
 
+    def eval_many(self, names):
+        """Several named tensors from ONE run of the graph: {name: flat float32 array}."""
+        outs = []
+        for what in names:
+            n = C.c_long()
+            _check(self.lib.dg_eval(self.h, what.encode(), None, C.byref(n)))
+            outs.append(np.empty(max(n.value, 1), np.float32))
+        ptrs = (_fp * len(outs))(*[_p(a) for a in outs])
+        _check(self.lib.dg_eval_many(self.h, ";".join(names).encode(), ptrs, len(outs)))
+        return dict(zip(names, outs))
+
+    @staticmethod
+    def grad_name(loss, name):
+        return "grad:%s:%s" % (loss, "x_fake" if name == "x_fake" else VAR_NAMES.index(name))
+
     def grad(self, loss, name):
         if name == "x_fake":
             return self.eval("grad:%s:x_fake" % loss, (self.batch, 64, 64, 3))
@@ -185,6 +204,13 @@ class DcganModel:
 
     def load_state(self, path):
         _check(self.lib.dg_load_state(self.h, path.encode()))
+
+
+def npz_inspect(path):
+    """(arrays, elements) of a .npz archive as the library's own reader sees it; HostError if it refuses the file."""
+    a, n = C.c_long(), C.c_long()
+    _check(load().dg_npz_inspect(path.encode(), C.byref(a), C.byref(n)))
+    return a.value, n.value
 
 
 def images_normalize(pix):

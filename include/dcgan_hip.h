@@ -52,13 +52,16 @@ int dh_device_info(char* name, size_t name_len, int* compute_units, int* clock_k
 /* tensor_alloc / tensor_free in GPU mode: src/memory/alloc.cu:16-37 (cudaMalloc / cudaFree). */
 int dh_malloc(void** ptr, size_t bytes);
 int dh_free(void* ptr);
-/* tensor_write / tensor_read in GPU mode: src/memory/copy.hxx:29-46 (blocking cudaMemcpy). */
+/* tensor_write / tensor_read in GPU mode: src/memory/copy.hxx:29-46 (blocking cudaMemcpy).  Like the
+ * reference's, these copies are ordered against the DEFAULT stream only; a caller that runs kernels on
+ * a stream of its own (dh_stream_create) waits for that stream before it copies results back. */
 int dh_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
 /* The same for the inputs a training loop feeds before every run (src/ops/graph.cu:139-147 writes each
  * fed input with tensor_write): the host buffer is copied into a pinned staging buffer of the library
  * (16 of them, used in turn) and from there to the device in `stream` order, so src_host may be
  * reused on return and kernels queued on `stream` afterwards see the data -- but the call does not
- * wait for the work queued before it, as the blocking copy does.  Copies above 64 MiB are blocking. */
+ * wait for the work queued before it, as the blocking copy does.  Copies above 64 MiB wait for
+ * `stream` and are then blocking. */
 int dh_memcpy_h2d_staged(void* dst_device, const void* src_host, size_t bytes, void* stream);
 int dh_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
 int dh_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
@@ -84,13 +87,31 @@ int dh_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop`
 int dh_workspace_reserve(size_t bytes);
 size_t dh_workspace_bytes(void);
 
+/* Pooled device memory for tensors: what tensor_alloc / tensor_free call in place of the reference's
+ * cudaMalloc / cudaFree per tensor (src/memory/alloc.cu:16-37; one per operator output at every
+ * Op::compile, src/ops/conv2d.cu:49-79, and again after an input changes shape, src/ops/graph.cu:104-120).
+ * Blocks are carved from a few large slabs the library keeps (256-byte aligned; freed neighbours merge),
+ * so a training loop -- and a recompile at another shape that fits what is held -- makes no hipMalloc or
+ * hipFree.  A freed block may be handed out again at once: correct for callers that queue all work on one
+ * stream (the stream orders the old tensor's last use before the new one's first); others synchronise or
+ * order their streams before freeing.  dh_pool_reserve makes sure that at least `bytes` are held and
+ * idle, dh_pool_trim returns idle slabs to the driver (after a device synchronisation), dh_pool_stats
+ * reports hipMalloc calls made so far, bytes held, bytes handed out and their peak (any may be NULL). */
+int dh_pool_alloc(void** ptr, size_t bytes);
+int dh_pool_free(void* ptr);
+int dh_pool_reserve(size_t bytes);
+int dh_pool_trim(void);
+int dh_pool_stats(size_t* hipmalloc_calls, size_t* bytes_held, size_t* bytes_in_use, size_t* peak_in_use);
+
 /* Per-kernel timing (no counterpart in the reference, whose only timer is the per-run wall clock of
  * src/ops/graph.cu:150-169).  on = 1 brackets the launches of the convolution kernels by HIP events
  * on the stream they are launched on; on = 2 also those of the reduction, dense and element-wise
  * kernels (some 150 launches per training iteration: the events then slow the iteration itself).
  * dh_profile_read() waits for them and writes one line per kernel tag:
- * "name<TAB>launches<TAB>total ms<TAB>total algorithmic work", the work being FLOPs, or bytes for
- * the memory-bound kernels, whose tags start with "hbm:". */
+ * "name<TAB>launches<TAB>total ms<TAB>total algorithmic work<TAB>total issued FLOPs", the work being
+ * FLOPs, or bytes for the memory-bound kernels, whose tags start with "hbm:"; the last column is what
+ * the matrix cores were issued for the convolution launches (live k-slabs as full tiles: skipped
+ * padding taps are not in it, the padding of partial tiles is), 0 where that is not accounted. */
 int dh_profile_enable(int on);
 int dh_profile_reset(void);
 int dh_profile_read(char* buf, size_t buf_len);

@@ -10,6 +10,41 @@ import numpy as np
 RTOL, ATOL = 1e-4, 1e-5
 
 
+def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
+    """The two-sided parity check of the batch-64 suites.  `exp32` is the oracle's fp32 result (the
+    reference's arithmetic and summation order), `exp64` the same computed with float64 sums.
+      * element by element: |got - exp32| <= 1e-4 |exp32| + 1e-5 max(1, max|exp32|) -- the stated fp32
+        tolerance, its absolute part widened for tensors of large magnitude (sums of thousands of O(1)
+        products cannot be held to 1e-5 by any fp32 summation order);
+      * against the float64 result, with the oracle's own fp32 rounding error as the yardstick:
+        max |got - exp64| <= max(2 * slack * max |exp32 - exp64|, 1e-5 * min(1, max|exp32|)) -- the
+        floor follows the magnitude downwards, so that gradients of magnitude 1e-6 are not waved
+        through by an absolute 1e-5.
+    slack = 3 for results downstream of an input-gradient product: there the reference adds blocks of
+    up to ceil(5/2)^2 = 9 products to its running sum (src/cpu/ops.hxx:651-672), which makes its fp32
+    error about sqrt(9) smaller than that of a kernel adding the same products one by one.
+    kinks: the tensor is a gradient through relu / leaky-relu layers.  A pre-activation within rounding
+    distance of zero takes either slope, depending on the summation order that produced it, and the
+    gradients downstream then differ by that element's whole contribution (measured between the batch-64
+    and the batch-512 kernels on the same images: 1 element of 4 194 304 in one generator layer, 1 of
+    2 097 152 in another, none elsewhere -- and three bias / filter gradients off by 1.4e-4 to 3.9e-4 of
+    their largest value in single entries).  Such tensors are allowed 2e-3 of their largest magnitude in
+    the float64 check, and their relative L2 error is held to 1e-3."""
+    got, exp32, exp64 = (np.asarray(a, np.float64).reshape(-1) for a in (got, exp32, exp64))
+    mag = float(np.abs(exp32).max()) if exp32.size else 0.0
+    yard = float(np.abs(exp32 - exp64).max()) if exp32.size else 0.0
+    err = float(np.abs(got - exp64).max()) if exp32.size else 0.0
+    print("%-50s max|exp| %.3g  oracle32-f64 %.3g  gpu-f64 %.3g  ratio %.2f" % (what, mag, yard, err, err / max(yard, 1e-30)),
+          flush=True)
+    if elementwise:
+        np.testing.assert_allclose(got, exp32, rtol=RTOL, atol=ATOL * max(1.0, mag), err_msg=what)
+    if kinks and exp32.size:
+        l2 = float(np.linalg.norm(got - exp64) / max(np.linalg.norm(exp64), 1e-30))
+        assert l2 <= 1e-3, "%s: relative L2 error %.3g" % (what, l2)
+    assert err <= max(2.0 * slack * yard, ATOL * min(1.0, mag), 2e-3 * mag if kinks else 0.0), \
+        "%s: max |gpu - f64| = %.3g, the oracle's own fp32 error is %.3g (max |exp| = %.3g)" % (what, err, yard, mag)
+
+
 def get(case, key, kind="inputs"):
     a = case[kind][key]
     return np.array(a["data"], dtype=np.float64).reshape(a["shape"])

@@ -3,7 +3,7 @@ of the reference DCGAN (dcgan/main.cu:89-120, :217-249, :304-307) used to pin th
 differentiation, and a script mode that evaluates the network through the host library in
 RT_MODE=CPU (the oracle as backend) and dumps everything to an .npz for the GPU parity test.
 
-    python tests/dcgan_reference.py <batch> <seed> <out.npz>
+    python tests/dcgan_reference.py <batch> <seed> <out.npz> [<iterations> [f64]]
 """
 import os
 import sys
@@ -31,23 +31,29 @@ def synthetic(batch, seed, shapes):
     return w, z, x
 
 
-def collect(model, steps=1):
-    """Everything the parity test compares, from a DcganModel with weights and inputs set."""
-    out = {}
-    for i in range(5):
-        out["g_l%d" % i] = model.eval("g_l%d" % i)
-    out["g_out"] = model.eval("g_out")
+def tensor_names():
+    """(key in the dump, name the facade's dg_eval understands) of everything the parity tests compare."""
+    import __graft_entry__ as ge
+    M = ge.load_package().hostabi.DcganModel
+    names = [("g_l%d" % i, "g_l%d" % i) for i in range(5)] + [("g_out", "g_out")]
     for br in ("d_fake", "d_real"):
-        for i in range(4):
-            out["%s_l%d" % (br, i)] = model.eval("%s_l%d" % (br, i))
-        out[br + "_logits"] = model.eval(br + "_logits")
-    for name in ("g_loss", "d_loss", "d_fake_loss", "d_real_loss"):
-        out[name] = model.eval(name)
-    for v in D_VARS:
-        out["grad_d_loss_" + v] = model.grad("d_loss", v).reshape(-1)
-    for v in G_VARS:
-        out["grad_g_loss_" + v] = model.grad("g_loss", v).reshape(-1)
-    out["grad_g_loss_x_fake"] = model.grad("g_loss", "x_fake").reshape(-1)
+        names += [("%s_l%d" % (br, i),) * 2 for i in range(4)] + [(br + "_logits",) * 2]
+    names += [(n, n) for n in ("g_loss", "d_loss", "d_fake_loss", "d_real_loss")]
+    names += [("grad_d_loss_" + v, M.grad_name("d_loss", v)) for v in D_VARS]
+    names += [("grad_g_loss_" + v, M.grad_name("g_loss", v)) for v in G_VARS + ["x_fake"]]
+    return names
+
+
+def collect(model, steps=1, one_run=True):
+    """Everything the parity test compares, from a DcganModel with weights and inputs set: every
+    layer, loss and gradient on the unchanged parameters (one run of the graph for all of them, or
+    one run per tensor), then `steps` iterations (D step, G step) and the parameters after them."""
+    names = tensor_names()
+    if one_run:
+        got = model.eval_many([n for _, n in names])
+        out = {key: got[n] for key, n in names}
+    else:
+        out = {key: model.eval(n) for key, n in names}
     losses = []
     for _ in range(steps):
         losses.append(model.d_step())
@@ -121,7 +127,8 @@ def main():
     steps = int(sys.argv[4]) if len(sys.argv) > 4 else 1
     import __graft_entry__ as ge
     pkg = ge.load_package()
-    backend = os.path.join(ROOT, "oracle", "liboracle_backend.so")
+    f64 = len(sys.argv) > 5 and sys.argv[5] == "f64"
+    backend = os.path.join(ROOT, "oracle", "liboracle_backend_f64.so" if f64 else "liboracle_backend.so")
     model = pkg.hostabi.DcganModel(batch, seed, "CPU", backend)
     w, z, x = synthetic(batch, seed, pkg.hostabi.var_shapes())
     for name, val in w.items():

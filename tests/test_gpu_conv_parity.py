@@ -404,8 +404,9 @@ def test_paired_launches(be, orc, shape):
 
 @pytest.mark.parametrize("shape", [(64, 32, 32, 64, 5, 5, 128, 2), (64, 16, 16, 128, 5, 5, 256, 2), (64, 8, 8, 256, 5, 5, 512, 2)])
 def test_paired_launches_at_batch_64_match_the_single_launches(be, shape):
-    """At the benchmark's shapes (too large for the CPU oracle in a test) the paired launches are
-    compared with the single launches, which the tests above tie to the oracle."""
+    """At the benchmark's shapes, on inputs in the benchmark's distributions, with a fused epilogue: the
+    paired launches against the single launches (test_gpu_layers_batch64.py compares both with the oracle
+    at these shapes on standard-normal inputs)."""
     import __graft_entry__ as ge
     A = ge.load_package().hipabi
     print("shape", shape, flush=True)
@@ -451,8 +452,8 @@ def test_dk_is_reproducible(be):
 
 
 def test_adjoint_at_full_batch(be):
-    """Size-independent check at the benchmark's batch 64 (where the CPU oracle would take minutes):
-    <conv(x,k), dy> = <x, dx(dy,k)> = <k, dk(x,dy)> for layer D2."""
+    """Size-independent check at the benchmark's batch 64, beside the oracle comparison of
+    test_gpu_layers_batch64.py: <conv(x,k), dy> = <x, dx(dy,k)> = <k, dk(x,dy)> for layer D2."""
     shape = (64, 16, 16, 128, 5, 5, 256, 2)
     x, k, dy = rand_conv_inputs(9, *shape)
     y = be.conv2d(x, k, (2, 2)).astype(np.float64)

@@ -1,7 +1,10 @@
 """Whole-network parity, layer by layer, in the manner of the reference's test_dcgan_generator /
-test_dcgan_discriminator (which export every layer, the loss and all dW/db): the DCGAN evaluated
-through the operator graph on the HIP backend against the same graph on the CPU oracle backend,
-on identical seeded weights and inputs -- unfused and with the fused launches."""
+test_dcgan_discriminator (tests/test_dcgan_discriminator.cu:49-136: every layer, the loss and all
+dW/db exported): the DCGAN evaluated through the operator graph on the HIP backend against the same
+graph on the CPU oracle backend, on identical seeded weights and inputs -- unfused and with the fused
+launches; at batch 2, and at the benchmark's batch 64 with three training iterations, where the
+float64-accumulating twin of the oracle gives the yardstick (the oracle's own fp32 error); the
+batch-512 iteration is tied to the batch-64 one through eight copies of its inputs."""
 import os
 import subprocess
 import sys
@@ -10,7 +13,7 @@ import numpy as np
 import pytest
 
 import dcgan_reference as dr
-from common import RTOL, ATOL
+from common import RTOL, ATOL, agree
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -26,20 +29,39 @@ def cpu_dump(tmp_path_factory):
     return dict(np.load(path))
 
 
-def gpu_dump(fusion):
+def oracle_dump(tmp_path_factory, batch, steps, f64=False):
+    path = str(tmp_path_factory.mktemp("dcgan") / ("cpu%d%s.npz" % (batch, "_f64" if f64 else "")))
+    env = dict(os.environ, RT_MODE="CPU", OMP_NUM_THREADS="16")
+    subprocess.run([sys.executable, os.path.join(ROOT, "tests", "dcgan_reference.py"), str(batch), str(SEED), path,
+                    str(steps)] + (["f64"] if f64 else []), check=True, env=env, timeout=900)
+    return dict(np.load(path))
+
+
+@pytest.fixture(scope="module")
+def cpu_dump64(tmp_path_factory):
+    return oracle_dump(tmp_path_factory, 64, 3)
+
+
+@pytest.fixture(scope="module")
+def cpu_dump64_f64(tmp_path_factory):
+    return oracle_dump(tmp_path_factory, 64, 3, f64=True)
+
+
+def gpu_dump(fusion, batch=BATCH, steps=1, one_run=False, tile=1):
     """fusion: False (one launch per instruction), True (fused launches, the two discriminator towers'
-    convolutions paired), "unpaired" (fused launches, every convolution on its own)."""
+    convolutions paired), "unpaired" (fused launches, every convolution on its own).  tile > 1: the
+    model runs at tile * batch with the batch's inputs repeated tile times."""
     import __graft_entry__ as ge
     pkg = ge.load_package()
-    model = pkg.hostabi.DcganModel(BATCH, SEED, "GPU")
+    model = pkg.hostabi.DcganModel(batch * tile, SEED, "GPU")
     try:
         model.set_fusion(bool(fusion))
         model.set_pairing(fusion != "unpaired")
-        w, z, x = dr.synthetic(BATCH, SEED, pkg.hostabi.var_shapes())
+        w, z, x = dr.synthetic(batch, SEED, pkg.hostabi.var_shapes())
         for name, val in w.items():
             model.set_var(name, val)
-        model.set_inputs(z, x)
-        return dr.collect(model), model.last_schedule_size()
+        model.set_inputs(np.tile(z, (tile, 1)), np.tile(x, (tile, 1, 1, 1)))
+        return dr.collect(model, steps, one_run), model.last_schedule_size()
     finally:
         model.set_fusion(False)
         model.set_pairing(True)
@@ -87,6 +109,78 @@ def test_dcgan_layers_losses_gradients_and_one_adam_iteration(cpu_dump, fusion):
         else:
             scale = max(1.0, float(np.abs(exp).max()))
             np.testing.assert_allclose(g, exp, rtol=RTOL, atol=ATOL * scale, err_msg=key)
+
+
+def agree_with_yardstick(key, got, exp32, exp64):
+    """common.agree with slack 3 (every tensor of the network lies downstream of an input-gradient
+    product).  Parameters after Adam steps additionally: a step is ~ lr * sign(gradient) while the second
+    moment is young, so a gradient at the rounding level flips the step of single elements in either
+    fp32 run (the yardstick then is a whole step); such elements must be as rare as in the oracle's own
+    fp32 run."""
+    agree(got, exp32, exp64, key, slack=3.0, elementwise=not key.startswith("after_"), kinks=key.startswith("grad_"))
+    if key.startswith("after_"):
+        got, exp32, exp64 = (np.asarray(a, np.float64).reshape(-1) for a in (got, exp32, exp64))
+        frac = float(np.mean(np.abs(got - exp64) > 1e-6))      # a step is 2e-4
+        frac32 = float(np.mean(np.abs(exp32 - exp64) > 1e-6))
+        print("%-50s moved differently: gpu %.3g, oracle32 %.3g of the elements" % (key, frac, frac32), flush=True)
+        assert frac <= 2.0 * frac32 + 1e-4, "%s: %.3g of the elements moved differently (oracle fp32: %.3g)" % (key, frac, frac32)
+
+
+@pytest.mark.parametrize("fusion", [True, False])
+def test_training_iterations_at_batch_64(cpu_dump64, cpu_dump64_f64, fusion):
+    """The benchmarked configuration: every layer of both networks, the four losses, all 21 gradients
+    (one run of the graph for all of them), then three training iterations (D step, G step; with
+    fusion: fused epilogues, paired towers, one optimiser launch per step) and every parameter after
+    them, against the oracle backend on the same inputs."""
+    print("fusion", fusion, flush=True)
+    got, _ = gpu_dump(fusion, batch=64, steps=3, one_run=True)
+    assert set(got) == set(cpu_dump64)
+    for key in sorted(cpu_dump64):
+        agree_with_yardstick(key, got[key], cpu_dump64[key], cpu_dump64_f64[key])
+
+
+def test_fused_plans_at_batch_64_tensor_by_tensor(cpu_dump64, cpu_dump64_f64):
+    """The same at batch 64 with one run of the graph PER requested tensor, so that everything upstream
+    of it runs in its fused, paired form (a tensor that is asked for is never fused away)."""
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    model = pkg.hostabi.DcganModel(64, SEED, "GPU")
+    try:
+        model.set_fusion(True)
+        w, z, x = dr.synthetic(64, SEED, pkg.hostabi.var_shapes())
+        for name, val in w.items():
+            model.set_var(name, val)
+        model.set_inputs(z, x)
+        names = dict(dr.tensor_names())
+        for key in ("g_out", "d_fake_l3", "d_real_logits", "d_loss", "g_loss", "grad_d_loss_d0_w", "grad_d_loss_d3_w",
+                    "grad_d_loss_d2_b", "grad_g_loss_g1_w", "grad_g_loss_g4_w", "grad_g_loss_g0_b", "grad_g_loss_x_fake"):
+            agree_with_yardstick(key, model.eval(names[key]), cpu_dump64[key], cpu_dump64_f64[key])
+    finally:
+        model.set_fusion(False)
+        model.close()
+
+
+def test_iteration_at_batch_512_repeats_the_batch_64_one(cpu_dump64, cpu_dump64_f64):
+    """The scaled configuration, batch 512, on eight copies of the oracle-checked batch-64 inputs: every
+    layer output repeats image by image, the mean losses and every parameter gradient equal the
+    batch-64 ones, and so do the parameters after three fused, paired training iterations."""
+    got, _ = gpu_dump(True, batch=64, steps=3, one_run=True, tile=8)
+    per_image = {"g_l0": 8192, "g_l1": 16384, "g_l2": 32768, "g_l3": 65536, "g_l4": 12288, "g_out": 12288,
+                 "grad_g_loss_x_fake": 12288}
+    for br in ("d_fake", "d_real"):
+        per_image.update({br + "_l0": 65536, br + "_l1": 32768, br + "_l2": 16384, br + "_l3": 8192, br + "_logits": 1})
+    for key in sorted(cpu_dump64):
+        g = got[key]
+        if key in per_image:
+            g = g.reshape(8, 64 * per_image[key])
+            for rep in range(1, 8):
+                np.testing.assert_allclose(g[rep], g[0], rtol=RTOL, atol=ATOL * max(1.0, float(np.abs(g[0]).max())),
+                                           err_msg="%s, copy %d" % (key, rep))
+            g = g[0]
+            if key == "grad_g_loss_x_fake":   # gradient of a mean over 8 times the images
+                agree_with_yardstick(key, g, cpu_dump64[key] / 8.0, cpu_dump64_f64[key] / 8.0)
+                continue
+        agree_with_yardstick(key, g, cpu_dump64[key], cpu_dump64_f64[key])
 
 
 def test_generate_and_argmax_bit_exact(cpu_dump):
