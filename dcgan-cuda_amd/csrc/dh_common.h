@@ -22,6 +22,10 @@ constexpr int MAX_ARENAS = 8;
 constexpr int STAGE_SLOTS = 16;                       // pinned staging buffers of dh_memcpy_h2d_staged
 constexpr size_t STAGE_MAX_BYTES = size_t(64) << 20;  // larger copies are plain blocking copies
 int workspace(size_t bytes, void** ptr, hipStream_t stream);
+// The current device's fixed scratch buffer (STATIC_SCRATCH_BYTES, part of the code object, never
+// allocated or freed): for entry points that must not allocate.  Every call on a device shares it.
+constexpr size_t STATIC_SCRATCH_BYTES = size_t(2) << 20;
+int static_scratch(void** ptr);
 int num_cus();
 
 // Per-kernel timing (see dh_profile_enable): prof_begin records an event on `st` and returns a

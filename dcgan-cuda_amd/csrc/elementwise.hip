@@ -404,8 +404,10 @@ ColsumCut colsum_cut(size_t rows, size_t cols)
 }
 
 // db: the column sums (both stages).  parts_out: the per-range sums of stage 1 only, left to the caller.
+// fixed_scratch: the row-range sums go to the device's fixed buffer instead of the stream's arena (no
+// allocation; the call is refused when they do not fit).
 int run_colsum(const char* who, const float* a, const float* act_ref, float* dz, float* db, float* parts_out,
-               size_t rows, size_t cols, ActGrad g, bool fused, void* stream)
+               size_t rows, size_t cols, ActGrad g, bool fused, void* stream, bool fixed_scratch = false)
 {
     DH_TRY(ensure_init());
     if (cols == 0) return 0;
@@ -431,12 +433,21 @@ int run_colsum(const char* who, const float* a, const float* act_ref, float* dz,
     else if (db && !partial)
     {
         void* ws;
-        DH_TRY(workspace(cut.chunks * cols * sizeof(float), &ws, st));
+        const size_t need = cut.chunks * cols * sizeof(float);
+        if (fixed_scratch)
+        {
+            if (need > STATIC_SCRATCH_BYTES)
+                return fail(DH_EINVAL, "%s: %zu x %zu needs %zu bytes of scratch, the fixed buffer holds %zu", who, rows,
+                            cols, need, STATIC_SCRATCH_BYTES);
+            DH_TRY(static_scratch(&ws));
+        }
+        else
+            DH_TRY(workspace(need, &ws, st));
         partial = static_cast<float*>(ws);
     }
     dim3 grid(cut.col_tiles, (unsigned)cut.chunks);
     ProfScope prof(fused ? "hbm:activation gradient + column sums (12 B/elem)" : "hbm:column sums (4 B/elem)",
-                   (fused ? 12.0 : 4.0) * rows * cols, st);
+                   (fused ? 12.0 : 4.0) * rows * cols, st, fixed_scratch ? 1 << 20 : 2);   // no events without allocating
     const bool al = aligned16(a) && (!fused || (aligned16(act_ref) && aligned16(dz)));
 #define DH_COLSUM_LAUNCH(KERNEL) \
     hipLaunchKernelGGL(KERNEL, grid, dim3(TPB), 0, st, a, act_ref, dz, partial, rows, (uint32_t)cols, cut.G, cut.rows_per_chunk, g)
@@ -745,6 +756,15 @@ int dh_bias_grad(const float* dz, float* db, size_t rows, size_t cols, void* str
     if (!db && cols) return fail(DH_EINVAL, "dh_bias_grad: null result");
     return run_colsum("dh_bias_grad", dz, nullptr, nullptr, db, nullptr, rows, cols, ActGrad{DH_ACT_NONE, 0.f}, false, stream);
 }
+
+int dh_bias_grad_static(const float* dz, float* db, size_t rows, size_t cols, void* stream)
+{
+    if (!db && cols) return fail(DH_EINVAL, "dh_bias_grad_static: null result");
+    return run_colsum("dh_bias_grad_static", dz, nullptr, nullptr, db, nullptr, rows, cols, ActGrad{DH_ACT_NONE, 0.f}, false,
+                      stream, true);
+}
+
+size_t dh_bias_grad_static_max_bytes(void) { return STATIC_SCRATCH_BYTES; }
 
 size_t dh_bias_grad_part_count(size_t rows, size_t cols)
 {

@@ -13,6 +13,11 @@ namespace
 {
 thread_local char g_err[512] = "";
 
+// Scratch of the entry points that must not allocate (dh_bias_grad_static): a fixed array in the
+// code object, one copy per GPU.  Host code never uses this name as an address: init_device asks
+// the runtime where the current device keeps its copy and stores that pointer in the device state.
+__attribute__((used)) static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
 struct DeviceState
 {
     bool ready = false;
@@ -27,6 +32,7 @@ struct DeviceState
     struct Stage { void* host; size_t bytes; hipEvent_t done; bool in_flight; };
     Stage stage[STAGE_SLOTS] = {};
     int next_stage = 0;
+    void* static_scratch = nullptr;   // this device's copy of `scratch`
 };
 
 std::mutex g_mu;
@@ -62,6 +68,9 @@ static int init_device(int device)
         if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
             return fail(DH_EINVAL, "dh_init: device %d is %s; this library holds gfx950 code only",
                         device, prop.gcnArchName);
+        void* fixed = nullptr;
+        DH_HIP(hipGetSymbolAddress(&fixed, HIP_SYMBOL(scratch)));
+        st.static_scratch = fixed;
         st.device = device;
         st.cus = prop.multiProcessorCount;
         st.ready = true;
@@ -80,6 +89,15 @@ int ensure_init()
 int num_cus()
 {
     return g_cur >= 0 ? g_dev[g_cur].cus : 256;
+}
+
+int static_scratch(void** ptr)
+{
+    DH_TRY(ensure_init());
+    *ptr = g_dev[g_cur].static_scratch;
+    if (!*ptr)
+        return fail(DH_EINVAL, "the fixed scratch buffer of device %d has no address", g_cur);
+    return 0;
 }
 
 int workspace(size_t bytes, void** ptr, hipStream_t stream)

@@ -60,6 +60,7 @@ _SIGS = {
     "dh_bias_add": [_vp, _vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad": [_vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad_parts": [_vp, _vp, _sz, _sz, _vp],
+    "dh_bias_grad_static": [_vp, _vp, _sz, _sz, _vp],
     "dh_mat_sum_rows": [_vp, _vp, _sz, _sz, _vp],
     "dh_relu": [_vp, _vp, _sz, _vp],
     "dh_relu_leaky": [_vp, _vp, _sz, _f, _vp],
@@ -89,6 +90,7 @@ _SIGS = {
 }
 # name -> result type, or (result type, argtypes)
 _RESTYPES = {"dh_version": C.c_char_p, "dh_last_error": C.c_char_p, "dh_workspace_bytes": _sz,
+             "dh_bias_grad_static_max_bytes": _sz,
              "dh_bias_grad_part_count": (_sz, [_sz, _sz])}
 
 _lib = None

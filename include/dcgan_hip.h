@@ -204,6 +204,18 @@ int dh_bias_grad(const float* dz, float* db, size_t rows, size_t cols, void* str
  * mat_sum_cols is one kernel per column block, src/gpu/sum.cu:112-151). */
 size_t dh_bias_grad_part_count(size_t rows, size_t cols);
 int dh_bias_grad_parts(const float* dz, float* parts, size_t rows, size_t cols, void* stream);
+/* dh_bias_grad for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same kernels, same
+ * summation order and bit-identical result, but the row-range sums go to a fixed buffer that is part
+ * of the library's code object instead of the stream's growing arena: the call allocates and frees
+ * nothing.  The buffer is dh_bias_grad_static_max_bytes() = 2 MiB per GPU, held until the process
+ * ends; every bias gradient of the DCGAN fits at any batch size.  The call fails with DH_EINVAL when
+ * dh_bias_grad_part_count(rows, cols) * cols floats exceed the buffer.  Every call on a GPU shares
+ * that GPU's buffer (each range sum is written before it is read, so nothing needs clearing): calls
+ * that overlap on one GPU -- from different streams or threads -- race; calls on one stream are
+ * ordered by the stream. */
+int dh_bias_grad_static(const float* dz, float* db, size_t rows, size_t cols, void* stream);
+size_t dh_bias_grad_static_max_bytes(void);
 /* out[r] = sum_c a[r,c].  Replaces gpu::mat_sum_rows (src/gpu/sum.cu:69-108). */
 int dh_mat_sum_rows(const float* a, float* out, size_t rows, size_t cols, void* stream);
 /* Replace vect_relu / vect_relu_leaky (src/gpu/relu.cu:26-55), vect_sigmoid / vect_tanh
