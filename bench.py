@@ -45,6 +45,7 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; averages over the launches of
 # one kernel symbol), each scaled by the same counter's reading for the calibration copy.  The
 # summaries are kept under profiles/.  None = not measured.
+TRAFFIC_SOURCE = "profiles/bench_iteration_bs64_hbm_traffic.md"
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
     # launch-weighted over the single and the paired instantiation of a tag
     "conv_igemm_fast<dx,128x64>": 88.8e6,       # 9 single launches of 73.6 MB, 2 paired of 157.1 MB per iteration
@@ -93,20 +94,44 @@ def synthetic(batch, seed=1234):
     return weights, z, x
 
 
-def cpu_baseline(batch, budget_s=25.0):
-    """Times the reference's CPU operators (compiled from its own header into oracle/_ref) on one
-    core: conv2d, conv2d_input_grad, conv2d_kernel_grad on layer D1 at batch 8 (about 10 s of CPU
-    work), then extrapolates one iteration from the measured FLOP/s of each class."""
+def host_cpu():
+    """(model name, logical CPUs this process may run on) of the host."""
+    name = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                name = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return name, usable
+
+
+def cpu_baseline(batch):
+    """Times the reference's CPU operators (compiled from its own sources into oracle/_ref) on this host:
+    conv2d, conv2d_input_grad, conv2d_kernel_grad on layer D1 at batch 4, one thread (RT_MODE=CPU
+    arithmetic; about 6 s), and extrapolates one iteration from the measured FLOP/s of each class.
+    RT_MODE=MCPU: the reference's rt::optimize + cpu::ThreadPoolRunner on 18 independent nodes of the
+    same operators at batch 2, with its own 4 workers (src/ops/graph.cu:32) and with one worker per
+    host core this process may use (at most 16, the share of a one-GPU box)."""
     oracle = ge.load_oracle()
     kind = "reference" if oracle.have_ref() else "port"
     orc = oracle.Oracle("ref" if kind == "reference" else "orc")
     orc.set_threads(1)
+    cpu_name, usable = host_cpu()
     rng = np.random.default_rng(0)
     H, W, C, O = LAYERS[1]
-    n = 8
-    x = rng.uniform(-1, 1, (n, H, W, C)).astype(np.float32)
-    k = (rng.standard_normal((5, 5, C, O)) * 0.02).astype(np.float32)
-    dy = rng.uniform(-1, 1, (n, H // 2, W // 2, O)).astype(np.float32)
+
+    def operands(n):
+        return (rng.uniform(-1, 1, (n, H, W, C)).astype(np.float32), (rng.standard_normal((5, 5, C, O)) * 0.02).astype(np.float32),
+                rng.uniform(-1, 1, (n, H // 2, W // 2, O)).astype(np.float32))
+
+    n = 4
+    x, k, dy = operands(n)
     fl = conv_flops(n, LAYERS[1])
     rates = {}
     t0 = time.perf_counter()
@@ -120,31 +145,46 @@ def cpu_baseline(batch, budget_s=25.0):
     rates["dk"] = fl / (time.perf_counter() - t0)
     work = iteration_flops(batch)
     seconds = sum(work[c] / rates[c] for c in ("fwd", "dx", "dk")) + work["dense"] / rates["fwd"]
-    mcpu = None
-    if kind == "reference":
-        # RT_MODE=MCPU: the same three operators as one node list through the reference's
-        # rt::optimize + ThreadPoolRunner with its 4 workers.  Its optimiser leaves convolution
-        # nodes whole, so what MCPU gains is the overlap of independent nodes (here three; the
-        # iteration's backward pass has two to four per layer).
-        sequential = sum(fl / rates[c] for c in ("fwd", "dx", "dk"))
+    out = {"value": 1.0 / seconds, "unit": "iterations/s", "cores": 1, "kind": kind, "host_cpu": cpu_name,
+           "host_cores_usable": usable,
+           "sample": "reference cpu::conv2d / conv2d_input_grad / conv2d_kernel_grad on layer D1 "
+                     "([%d,32,32,64] -> 128, 5x5, s2) once each, one thread; iteration time extrapolated "
+                     "from the per-class GFLOP/s (%.3f / %.3f / %.3f) over %.0f GFLOP"
+                     % (n, rates["fwd"] / 1e9, rates["dx"] / 1e9, rates["dk"] / 1e9, work["total"] / 1e9),
+           "gflops": {c: rates[c] / 1e9 for c in rates}}
+    if kind != "reference":
+        return out
+    # RT_MODE=MCPU.  The reference's optimiser leaves convolution nodes whole (src/runtime/optimizer.cu:
+    # 239-247, 561-583): what its thread pool gains is the overlap of independent nodes, so the sample is
+    # a list of independent nodes -- 6 x (conv2d, input gradient, filter gradient) at batch 2 -- and the
+    # speedup over running that list on one thread is an upper bound for a training iteration, whose
+    # backward pass offers two to four independent nodes per layer.
+    n2, copies = 2, 6
+    fl2 = conv_flops(n2, LAYERS[1])
+    sequential = copies * sum(fl2 / rates[c] for c in ("fwd", "dx", "dk"))
+
+    def mcpu(workers):
         prog = oracle.RefProgram()
-        nodes = [prog.conv2d(x, k, (2, 2), (3, 3))[0], prog.conv2d_input_grad(dy, k, 2, (H, W))[0],
-                 prog.conv2d_kernel_grad(dy, x, 2, (3, 3))[0]]
+        nodes = []
+        for _ in range(copies):
+            x2, k2, dy2 = operands(n2)
+            nodes += [prog.conv2d(x2, k2, (2, 2), (3, 3))[0], prog.conv2d_input_grad(dy2, k2, 2, (H, W))[0],
+                      prog.conv2d_kernel_grad(dy2, x2, 2, (3, 3))[0]]
         t0 = time.perf_counter()
-        prog.run(nodes, mcpu=True, workers=4)
-        t_mcpu = time.perf_counter() - t0
-        mcpu = {"workers": 4, "sample_seconds": t_mcpu, "sequential_seconds": sequential,
-                "speedup": sequential / t_mcpu, "value": sequential / t_mcpu / seconds,
-                "unit": "iterations/s",
-                "sample": "the same three operators as independent nodes of one list, run by the "
-                          "reference's rt::optimize + cpu::ThreadPoolRunner(4); iteration rate = the "
-                          "one-thread rate x the measured speedup"}
-    return {"value": 1.0 / seconds, "unit": "iterations/s", "cores": 1, "kind": kind, "mcpu": mcpu,
-            "sample": "reference cpu::conv2d / conv2d_input_grad / conv2d_kernel_grad on layer D1 "
-                      "([8,32,32,64] -> 128, 5x5, s2) once each, one thread; iteration time extrapolated "
-                      "from the per-class GFLOP/s (%.3f / %.3f / %.3f) over %.0f GFLOP"
-                      % (rates["fwd"] / 1e9, rates["dx"] / 1e9, rates["dk"] / 1e9, work["total"] / 1e9),
-            "gflops": {c: rates[c] / 1e9 for c in rates}}
+        prog.run(nodes, mcpu=True, workers=workers)
+        t = time.perf_counter() - t0
+        return {"workers": workers, "sample_seconds": t, "speedup": sequential / t, "value": sequential / t / seconds,
+                "unit": "iterations/s"}
+
+    out["mcpu"] = mcpu(4)
+    out["mcpu_all_cores"] = mcpu(max(1, min(usable, 16)))
+    out["mcpu_value"] = out["mcpu"]["value"]
+    out["mcpu_all_cores_value"] = out["mcpu_all_cores"]["value"]
+    out["mcpu_all_cores_workers"] = out["mcpu_all_cores"]["workers"]
+    out["mcpu_sample"] = ("18 independent nodes (6 x conv2d / input gradient / filter gradient of D1 at batch 2) through the "
+                          "reference's rt::optimize + cpu::ThreadPoolRunner; %.1f s on one thread (from the per-class rates); "
+                          "iteration rate = one-thread rate x measured speedup, an upper bound" % sequential)
+    return out
 
 
 def calibration_copy(A):
@@ -183,6 +223,13 @@ def layer_sweep(args, A):
         }
         flops = conv_flops(N, (H, W, C, O))
         for name, fn in ops.items():
+            # one bracketed launch tells which kernel runs and what the matrix cores are issued for it
+            A.profile_reset()
+            A.profile_enable(1)
+            fn()
+            A.profile_enable(0)
+            tagged = A.profile_read()
+            issued = sum(r["issued"] for r in tagged) if tagged and all(r["issued"] > 0 for r in tagged) else None
             t.start()
             for _ in range(3):
                 fn()
@@ -197,7 +244,9 @@ def layer_sweep(args, A):
             ms = t.stop_ms() / reps
             tf = flops / (ms * 1e-3) / 1e12
             rows.append({"layer": "D%d" % li, "x": [N, H, W, C], "k": [5, 5, C, O], "op": name, "launches": reps,
-                         "us": round(ms * 1e3, 2), "tflops": round(tf, 2), "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4)})
+                         "kernel": "+".join(r["name"] for r in tagged),
+                         "us": round(ms * 1e3, 2), "tflops": round(tf, 2), "frac": round(tf / PEAK_FP32_MFMA_TFLOPS, 4),
+                         "issued_frac": round(issued / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4) if issued else None})
     heavy = [r for r in rows if r["layer"] != "D0"]
     total_fl = sum(conv_flops(N, LAYERS[int(r["layer"][1])]) for r in heavy)
     total_s = sum(r["us"] * 1e-6 for r in heavy)
@@ -212,8 +261,11 @@ def layer_sweep(args, A):
                                "operators of layers D1-D3 once each (D0 rows listed, not in value)" % N, "batch": N},
         "device": A.device_info(),
         "roofline": {"kernel": "%s %s" % (worst["layer"], worst["op"]), "bound": "mfma", "achieved": worst["tflops"],
-                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": worst["frac"], "traffic": None,
-                     "note": "the slowest of the nine operators; every row is in `layers`"},
+                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": worst["frac"],
+                     "issued_frac": worst["issued_frac"], "traffic": None,
+                     "note": "the slowest of the nine operators; every row is in `layers`; `frac` counts skipped "
+                             "padding products as work (it can exceed 1), `issued_frac` is what the matrix cores "
+                             "are issued per second against the peak (slice reduction inside the time of both)"},
         "layers": rows,
     }))
 
@@ -353,7 +405,9 @@ def generator_only(args, pkg, A):
                                           "ms_per_step": round(conv_ms / max(profiled, 1), 4)},
                      "kernels": [{"name": r["name"], "launches": r["launches"],
                                   "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
-                                  "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2)}
+                                  "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2),
+                                  "issued_frac": round(r["issued"] / (r["ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)
+                                  if r["issued"] > 0 else None}
                                  for r in sorted(rows, key=lambda r: -r["ms"])]},
     }))
     model.close()
@@ -399,8 +453,10 @@ def main():
     model.set_inputs(z, x)   # resident from here on
 
     def iteration():
-        if args.host_inputs:
-            model.set_inputs(z, x)   # blocking host-to-device copies, as the reference's Graph::run feeds its inputs
+        if args.host_inputs:         # inputs handed to the runs from pageable host memory, as the reference's loop does
+            model.d_step(want_loss=False, z=z, x=x)
+            model.g_step(want_loss=False, z=z)
+            return
         model.d_step(want_loss=False)
         model.g_step(want_loss=False)
 
@@ -445,6 +501,17 @@ def main():
     d_loss = model.eval("d_loss")[0]
     g_loss = model.eval("g_loss")[0]
 
+    # the reference's own loop (dcgan/main.cu:378-397): z and the image batch fed from host memory and
+    # both losses read back in every iteration -- reported beside the resident rate, never as `value`
+    ref_steps = max(1, min(args.steps, 50))
+    for _ in range(3):
+        model.d_step(z=z, x=x), model.g_step(z=z)
+    t1 = time.perf_counter()
+    for _ in range(ref_steps):
+        model.d_step(z=z, x=x)     # graph.run({d_opti, d_loss}, {z, x}) and the loss read back
+        model.g_step(z=z)          # graph.run({g_opti, g_loss}, {z}) and the loss read back
+    ref_wall = time.perf_counter() - t1
+
     calibration_copy(A)
 
     ms_per_step = wall * 1e3 / args.steps
@@ -456,19 +523,31 @@ def main():
     dom = max(rows, key=lambda r: r["ms"])
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
     traffic = MEASURED_TRAFFIC_BYTES.get(dom["name"]) if args.batch == 64 else None
+
+    def issued_frac(r):
+        """Matrix-core utilisation proper: the FLOPs the kernel issues (live k-slabs as full tiles --
+        skipped padding taps are not in it) per second against the peak.  The algorithmic `frac` counts
+        the skipped products as work done and may exceed it."""
+        return round(r["issued"] / (r["ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4) if r["issued"] > 0 else None
+
     roofline = {
         "kernel": dom["name"], "bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": traffic,
+        "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "issued_frac": issued_frac(dom),
+        "traffic": traffic, "traffic_source": TRAFFIC_SOURCE if traffic else None,
         "launches": dom["launches"], "avg_launch_us": round(dom["ms"] * 1e3 / dom["launches"], 2),
         "flops_per_launch": dom["flops"] / dom["launches"],
+        "issued_flops_per_launch": dom["issued"] / dom["launches"] if dom["issued"] > 0 else None,
         "all_conv_kernels": {"tflops": round(conv_fl / (conv_ms * 1e-3) / 1e12, 3),
                              "frac": round(conv_fl / (conv_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
                              "ms_per_step": round(conv_ms / max(profiled, 1), 4)},
         "profiled_iterations": profiled,
         "kernels": [{"name": r["name"], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
-                     "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2)} for r in sorted(rows, key=lambda r: -r["ms"])],
+                     "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2),
+                     "frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                     "issued_frac": issued_frac(r)} for r in sorted(rows, key=lambda r: -r["ms"])],
         "hbm_kernels": [{"name": r["name"][4:], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
-                         "gbs": round(r["flops"] / (r["ms"] * 1e-3) / 1e9, 1),
+                         "bytes_per_launch": round(r["flops"] / r["launches"]),
+                         "gbs": round(r["flops"] / (r["ms"] * 1e-3) / 1e9, 3),
                          "frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                          "ms_per_step": round(r["ms"] / aux_steps, 4)} for r in sorted(hbm_rows, key=lambda r: -r["ms"])],
         "dense_gemm": [{"launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
@@ -489,6 +568,11 @@ def main():
         "iteration_gflop": round(work["total"] / 1e9, 2),
         "iteration_tflops": round(work["total"] / (wall / args.steps) / 1e12, 3),
         "losses_after": {"d_loss": float(d_loss), "g_loss": float(g_loss)},
+        "reference_loop_value": round(ref_steps / ref_wall, 3),
+        "reference_loop": {"value": round(ref_steps / ref_wall, 3), "unit": "iterations/s", "steps": ref_steps,
+                           "ms_per_step": round(ref_wall * 1e3 / ref_steps, 4),
+                           "what": "the reference's own training loop (dcgan/main.cu:378-397): z and the image batch fed "
+                                   "from pageable host memory and both losses read back in every iteration"},
         "device": A.device_info(),
         "roofline": roofline,
     }

@@ -50,10 +50,10 @@ void forget_plans();
 void set_sync_each_run(bool on);
 bool sync_each_run();
 
-// Copies `count` values from host memory into the device tensor at `dst` for the runs that follow: on a
-// copy stream of the backend's own, behind the work queued so far; the launch stream waits for the copy
-// in front of the first step that touches the tensor (or at the end of the next run).  src_host may be
-// reused on return.
+// Notes that the device tensor at `dst` is to receive `count` values from host memory before the next
+// run reads it.  The run stages and copies the data in front of the first step that touches the tensor
+// (after queueing the steps before it), or at its end; src_host must stay valid until that run -- or
+// hip::synchronize() -- returns.  Graph::run feeds its inputs this way.
 void feed(dbl_t* dst, const dbl_t* src_host, std::size_t count);
 
 void* stream();  // hipStream_t the backend launches on

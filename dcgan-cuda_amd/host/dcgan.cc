@@ -309,22 +309,39 @@ int dg_set_inputs(void* model, const float* z_host, const float* x_host)
     });
 }
 
-int dg_d_step(void* model, float* d_loss)
+namespace
+{
+std::map<ops::Input*, std::pair<const dbl_t*, ops::Shape>> fed(dcgan::Model& m, const float* z_host, const float* x_host)
+{
+    std::map<ops::Input*, std::pair<const dbl_t*, ops::Shape>> in;
+    if (z_host)
+        in[m.z] = {z_host, ops::Shape({m.batch, 100})};
+    if (x_host)
+        in[m.x] = {x_host, ops::Shape({m.batch, 64, 64, 3})};
+    return in;
+}
+}  // namespace
+
+int dg_d_step(void* model, float* d_loss) { return dg_d_step_fed(model, nullptr, nullptr, d_loss); }
+
+int dg_d_step_fed(void* model, const float* z_host, const float* x_host, float* d_loss)
 {
     return guarded([&] {
         dcgan::Model& m = M(model);
         hip::set_sync_each_run(d_loss != nullptr);
-        ops::Graph::instance().run({m.d_opti, m.d_loss}, {}, {nullptr, d_loss});
+        ops::Graph::instance().run({m.d_opti, m.d_loss}, fed(m, z_host, x_host), {nullptr, d_loss});
         hip::set_sync_each_run(true);
     });
 }
 
-int dg_g_step(void* model, float* g_loss)
+int dg_g_step(void* model, float* g_loss) { return dg_g_step_fed(model, nullptr, g_loss); }
+
+int dg_g_step_fed(void* model, const float* z_host, float* g_loss)
 {
     return guarded([&] {
         dcgan::Model& m = M(model);
         hip::set_sync_each_run(g_loss != nullptr);
-        ops::Graph::instance().run({m.g_opti, m.g_loss}, {}, {nullptr, g_loss});
+        ops::Graph::instance().run({m.g_opti, m.g_loss}, fed(m, z_host, nullptr), {nullptr, g_loss});
         hip::set_sync_each_run(true);
     });
 }

@@ -60,6 +60,11 @@ int dg_set_inputs(void* model, const float* z_host, const float* x_host);
 // is copied back and the call returns while the GPU is still running).
 int dg_d_step(void* model, float* d_loss);
 int dg_g_step(void* model, float* g_loss);
+// The same with the inputs handed to the run itself, as the reference's training loop does
+// (dcgan/main.cu:378-391: graph.run({opti, loss}, {{z, ...}, {x, ...}}, ...)); a NULL input stays as it is
+// on the device.  The buffers are borrowed until the call returns.
+int dg_d_step_fed(void* model, const float* z_host, const float* x_host, float* d_loss);
+int dg_g_step_fed(void* model, const float* z_host, float* g_loss);
 int dg_sync(void);
 // Generator forward only: images [batch,64,64,3] to host.
 int dg_generate(void* model, float* images_host);

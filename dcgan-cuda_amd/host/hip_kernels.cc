@@ -894,11 +894,11 @@ bool sync_each_run() { return g_sync_each_run; }
 
 void* stream() { return g_stream; }   // hip_table.hh: the default stream
 
-namespace { void wait_for_feeds(const Step* s); }
+namespace { void flush_feeds(const Step* s); }
 
 void synchronize()
 {
-    wait_for_feeds(nullptr);
+    flush_feeds(nullptr);
     CK(dh_stream_sync(g_stream));
 }
 
@@ -910,27 +910,16 @@ void set_protected_tensors(const std::vector<const dbl_t*>& tensors)
 
 // ---- inputs fed from host memory --------------------------------------------------------------
 // The reference copies every fed input with a blocking cudaMemcpy in front of the run
-// (src/ops/graph.cu:139-147), which first drains whatever is still executing.  Here the copy goes to a
-// stream of its own: it starts once the work queued so far has finished (an earlier run may still read
-// the tensor), and the launch stream waits for it only in front of the first step that touches the
-// tensor -- the image batch of a discriminator step arrives while the generator's forward pass runs.
+// (src/ops/graph.cu:139-147), which first drains whatever is still executing and leaves the GPU idle
+// while the host copies.  Here a fed input is only noted (feed); the run that follows stages and copies
+// it, in stream order, right in front of the first step that touches the tensor, after the steps before
+// it have been queued: the host stages the image batch of a discriminator step while the generator's
+// forward pass runs.  (Sending the copy through a second stream with events either side was measured
+// too: the two cross-stream waits per input cost more than the overlap of a 3 MB copy gains.)
 namespace
 {
-struct Feed { const dbl_t* begin; const dbl_t* end; void* done; };
-std::vector<Feed> g_feeds;             // copies the launch stream has not been ordered behind yet
-void* g_copy_stream = nullptr;
-constexpr int FEED_EVENTS = 32;        // ring of (queued-so-far, copy-done) event pairs
-void* g_feed_events[FEED_EVENTS] = {};
-int g_next_feed_event = 0;
-
-void* next_feed_event()
-{
-    void*& e = g_feed_events[g_next_feed_event];
-    g_next_feed_event = (g_next_feed_event + 1) % FEED_EVENTS;
-    if (!e)
-        CK(dh_event_create(&e));
-    return e;
-}
+struct Feed { dbl_t* begin; dbl_t* end; const dbl_t* src; };
+std::vector<Feed> g_feeds;             // noted, not yet copied
 
 bool node_touches(const rt::Node* n, const Feed& f)
 {
@@ -955,14 +944,20 @@ bool step_touches(const Step& s, const Feed& f)
     return false;
 }
 
-// Orders the launch stream behind every outstanding copy (all == true) or behind those `s` touches.
-void wait_for_feeds(const Step* s)
+void copy_now(const Feed& f)
+{
+    CK(dh_memcpy_h2d_staged(f.begin, f.src, (std::size_t)(f.end - f.begin) * sizeof(dbl_t), g_stream));
+}
+
+// Copies the noted inputs that step `s` touches (all of them when s is null).
+void flush_feeds(const Step* s)
 {
     for (std::size_t i = 0; i < g_feeds.size();)
         if (!s || step_touches(*s, g_feeds[i]))
         {
-            CK(dh_stream_wait_event(g_stream, g_feeds[i].done));
+            const Feed f = g_feeds[i];
             g_feeds.erase(g_feeds.begin() + (long)i);
+            copy_now(f);
         }
         else
             ++i;
@@ -973,23 +968,13 @@ void feed(dbl_t* dst, const dbl_t* src_host, std::size_t count)
 {
     if (count == 0)
         return;
-    if (!g_copy_stream)
-        CK(dh_stream_create(&g_copy_stream));
-    // an outstanding copy into the same tensor is ordered before this one by the copy stream itself
+    // a second feed of the same tensor replaces the first
     for (std::size_t i = 0; i < g_feeds.size();)
         if (g_feeds[i].begin < dst + count && dst < g_feeds[i].end)
             g_feeds.erase(g_feeds.begin() + (long)i);
         else
             ++i;
-    void* queued = next_feed_event();
-    void* done = next_feed_event();
-    CK(dh_event_record(queued, g_stream));
-    CK(dh_stream_wait_event(g_copy_stream, queued));
-    CK(dh_memcpy_h2d_staged(dst, src_host, count * sizeof(dbl_t), g_copy_stream));
-    CK(dh_event_record(done, g_copy_stream));
-    g_feeds.push_back(Feed{dst, dst + count, done});
-    if (g_feeds.size() > FEED_EVENTS / 4)   // far more inputs than a graph feeds: do not outrun the event ring
-        wait_for_feeds(nullptr);
+    g_feeds.push_back(Feed{dst, dst + count, src_host});
 }
 
 void run_async(rt::NodesList& tasks)
@@ -1002,11 +987,11 @@ void run_async(rt::NodesList& tasks)
     for (const Step& s : it->second.steps)
     {
         if (!g_feeds.empty())
-            wait_for_feeds(&s);
+            flush_feeds(&s);
         issue(s);
     }
-    // whatever the run did not touch: results are read back with copies that only see the launch stream
-    wait_for_feeds(nullptr);
+    // inputs the run did not touch: the caller's buffers are only borrowed until the run returns
+    flush_feeds(nullptr);
     g_last_launches = (int)it->second.steps.size();
 }
 

@@ -1,4 +1,7 @@
 #include "ops.hh"
+
+#include <cstdlib>
+#include <cstring>
 #include "npz.hh"
 
 #include <algorithm>
@@ -238,7 +241,9 @@ void Graph::run(std::vector<Op*> ops, const std::map<Input*, std::pair<const dbl
     {
         compile_(kv.first);
         dbl_t* dst = compiled(kv.first).out_data;
-        if (program_mode() == ProgramMode::GPU)
+        // DCGAN_HIP_FEED=front: the copy in front of the run, as the reference places it
+        static const bool deferred = !(std::getenv("DCGAN_HIP_FEED") && !std::strcmp(std::getenv("DCGAN_HIP_FEED"), "front"));
+        if (program_mode() == ProgramMode::GPU && deferred)
             hip::feed(dst, kv.second.first, (std::size_t)kv.second.second.total());
         else
             tensor_write(dst, dst + kv.second.second.total(), kv.second.first);

@@ -40,6 +40,8 @@ def load():
         lib.dg_set_inputs.argtypes = [C.c_void_p, _fp, _fp]
         lib.dg_d_step.argtypes = [C.c_void_p, _fp]
         lib.dg_g_step.argtypes = [C.c_void_p, _fp]
+        lib.dg_d_step_fed.argtypes = [C.c_void_p, _fp, _fp, _fp]
+        lib.dg_g_step_fed.argtypes = [C.c_void_p, _fp, _fp]
         lib.dg_generate.argtypes = [C.c_void_p, _fp]
         lib.dg_eval.argtypes = [C.c_void_p, C.c_char_p, _fp, C.POINTER(C.c_long)]
         lib.dg_eval_many.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(_fp), C.c_int]
@@ -135,14 +137,19 @@ class DcganModel:
         x = None if x is None else np.ascontiguousarray(x, np.float32)
         _check(self.lib.dg_set_inputs(self.h, _p(z) if z is not None else None, _p(x) if x is not None else None))
 
-    def d_step(self, want_loss=True):
+    def d_step(self, want_loss=True, z=None, x=None):
+        """One discriminator step; z / x (host arrays) are fed to the run itself when given."""
         loss = C.c_float()
-        _check(self.lib.dg_d_step(self.h, C.byref(loss) if want_loss else None))
+        z = None if z is None else np.ascontiguousarray(z, np.float32)
+        x = None if x is None else np.ascontiguousarray(x, np.float32)
+        _check(self.lib.dg_d_step_fed(self.h, None if z is None else _p(z), None if x is None else _p(x),
+                                      C.byref(loss) if want_loss else None))
         return loss.value if want_loss else None
 
-    def g_step(self, want_loss=True):
+    def g_step(self, want_loss=True, z=None):
         loss = C.c_float()
-        _check(self.lib.dg_g_step(self.h, C.byref(loss) if want_loss else None))
+        z = None if z is None else np.ascontiguousarray(z, np.float32)
+        _check(self.lib.dg_g_step_fed(self.h, None if z is None else _p(z), C.byref(loss) if want_loss else None))
         return loss.value if want_loss else None
 
     def sync(self):

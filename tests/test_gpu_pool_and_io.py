@@ -179,3 +179,37 @@ def test_images_from_files_into_a_discriminator_step(pkg, tmp_path, orc):
     finally:
         model.set_fusion(False)
         model.close()
+
+
+def test_inputs_handed_to_the_run_equal_resident_inputs(pkg):
+    """The reference's loop passes z and the image batch to every run (dcgan/main.cu:378-391); here such
+    inputs are staged and copied inside the run, in front of the first step that reads them.  Three
+    iterations fed that way -- with fresh inputs each time, losses read and not read -- against the same
+    iterations on inputs made resident beforehand: identical losses and parameters."""
+    H = pkg.hostabi
+    rng = np.random.default_rng(5)
+    batch = 16
+    zs = [rng.uniform(-1, 1, (batch, 100)).astype(np.float32) for _ in range(3)]
+    xs = [rng.uniform(-1, 1, (batch, 64, 64, 3)).astype(np.float32) for _ in range(3)]
+    results = []
+    for fed in (False, True):
+        model = make_model(pkg, batch)
+        try:
+            losses = []
+            for i, (z, x) in enumerate(zip(zs, xs)):
+                want = i != 1
+                if fed:
+                    zc, xc = z.copy(), x.copy()
+                    losses.append((model.d_step(want, z=zc, x=xc), model.g_step(want, z=zc)))
+                    zc[:], xc[:] = 7.0, 7.0      # the buffers are the caller's again once the call has returned
+                else:
+                    model.set_inputs(z, x)
+                    losses.append((model.d_step(want), model.g_step(want)))
+            results.append((losses, snapshot(model, H)))
+        finally:
+            model.set_fusion(False)
+            model.close()
+    assert results[0][0] == results[1][0]
+    assert all(np.isfinite(v) for pair in results[0][0] for v in pair if v is not None)
+    for n in H.VAR_NAMES:
+        np.testing.assert_array_equal(results[0][1][n], results[1][1][n], err_msg=n)
