@@ -176,8 +176,10 @@ __global__ __launch_bounds__(256) void dx_few_channels(const SmallDxParams p)
 // gathers into LDS.  Here the MFMA operands never pass through LDS: lane (m, h) of a wavefront owns
 // output pixel m of a 32-pixel tile and loads ITS patch values k = h*40 + j straight from global
 // memory into the register that MFMA number j consumes; the filter (at most 80 x 64 values) is
-// staged in LDS once per workgroup and read from there, one value per lane and MFMA.  A wavefront
-// computes one tile (two, with the second tile's loads in flight during the first's MFMAs, was slower).
+// staged in LDS once per workgroup and read from there, one value per lane and MFMA.  Workgroups are
+// persistent (two per compute unit, two wavefronts per SIMD): a wavefront walks over tiles with the
+// loads of its next tile issued before the MFMAs of the current one, so that one wavefront of a SIMD
+// multiplies while the other waits for memory or writes its tile out.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int TF_KH = 40;           // MFMAs per 32-output-channel block; the contraction is padded to 2 * TF_KH
@@ -194,6 +196,7 @@ struct ThinFwdParams
     int N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pt, pl;
     int K, row;             // kh*kw*C and kw*C (one filter row of taps)
     int pixels;             // N*Ho*Wo
+    int tiles;              // 32-pixel tiles
     uint32_t x_bytes;
     FastDiv fd_HoWo, fd_Wo, fd_row, fd_C;
 };
@@ -205,63 +208,59 @@ struct ThinFwdParams
 // replaced by zero after the load; the buffer descriptor's range check is per dword, so a load that
 // runs past the end of the tensor still delivers its in-range elements.
 template <bool ROWS>
-__global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
+__global__ __launch_bounds__(256, 2) void fwd_thin(const ThinFwdParams p)
 {
     __shared__ float filt[2 * TF_KH * 32 * TF_NB];   // [k][n], zero beyond K and O
+    __shared__ __attribute__((aligned(16))) float lbias[32 * TF_NB];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const float* bw = filt + half * TF_KH * (32 * TF_NB) + l32;   // + q * 64 + nb * 32
 
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
-    // The wavefront's one tile.  Its patch loads are issued before the filter is staged, so that the
-    // two round trips to memory overlap (a wavefront past the last tile loads nothing: every offset
-    // is out of range).
-    {
-        const int tile = blockIdx.x * 4 + wave;
-        const int pix = tile * 32 + l32;
-        const bool live = pix < p.pixels;
-        uint32_t b, rem, i, j;
-        p.fd_HoWo.divmod(live ? pix : 0, b, rem);
-        p.fd_Wo.divmod(rem, i, j);
-        const int h0 = (int)i * p.sh - p.pt, w0 = (int)j * p.sw - p.pl;
-        const int base = (((int)b * p.H + h0) * p.W + w0) * p.C * 4;
 
-        float a[TF_KH];
+    // Patch of this lane's pixel of `tile`, in two halves so that the round trip to memory lies behind
+    // the MFMAs of the tile before: issue() sends the loads (raw 16-byte pieces for ROWS, the values
+    // themselves otherwise; nothing is in range for a tile past the last one), finish() -- called when
+    // the values are needed -- replaces the elements that belong to no tap by zero.
+    struct Pixel { int h0, w0, base; bool live, corner; };
+    auto pixel_of = [&](int tile) {
+        const int pix = tile * 32 + l32;
+        Pixel px;
+        px.live = tile < p.tiles && pix < p.pixels;
+        uint32_t b, rem, i, j;
+        p.fd_HoWo.divmod(px.live ? pix : 0, b, rem);
+        p.fd_Wo.divmod(rem, i, j);
+        px.h0 = (int)i * p.sh - p.pt;
+        px.w0 = (int)j * p.sw - p.pl;
+        px.base = (((int)b * p.H + px.h0) * p.W + px.w0) * p.C * 4;
+        // Pixels of the first image whose patch has padding on its left and holds input row 0: the
+        // 16-byte load of that row would begin before the tensor (a negative offset, which the range
+        // check rejects as a whole, in-range elements included).  Those few pixels take 4-byte loads.
+        px.corner = px.live && b == 0 && px.h0 <= 0 && px.w0 < 0;
+        return px;
+    };
+    // per-lane constants of the ten 16-byte chunks: byte offset within the patch (far out of range for
+    // a chunk whose filter row does not exist) and filter row
+    constexpr int FAR = (int)0xC0000000u;     // + any patch offset stays above every tensor size (< 2 GiB)
+    int chunk_off[TF_KH / 4], chunk_di[TF_KH / 4];
+#pragma unroll
+    for (int u = 0; u < TF_KH / 4; ++u)
+    {
+        const int k0 = half * TF_KH + 4 * u;        // first k' of the chunk
+        const int di = k0 >> 4, t0 = k0 & 15;
+        chunk_di[u] = di;
+        chunk_off[u] = di < p.kh ? (di * p.W * p.C + t0) * 4 : FAR;
+    }
+    auto issue = [&](const Pixel& px, f32x4v (&raw)[TF_KH / 4], float (&a)[TF_KH]) {
         if (ROWS)
         {
+            const int base = px.live ? px.base : FAR;
 #pragma unroll
             for (int u = 0; u < TF_KH / 4; ++u)
             {
-                const int k0 = half * TF_KH + 4 * u;        // first k' of the chunk
-                const int di = k0 >> 4, t0 = k0 & 15;
-                const bool row_ok = (int)live & (int)(di < p.kh) & (int)((unsigned)(h0 + di) < (unsigned)p.H);
-                const int off = row_ok ? base + (di * p.W * p.C + t0) * 4 : (int)0x80000000u;
-                const f32x4v v = __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(xr, off, 0, 0));
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                {
-                    const int t = t0 + e;
-                    const int dj = (int)p.fd_C.div((uint32_t)t);
-                    const bool ok = (int)(t < p.row) & (int)((unsigned)(w0 + dj) < (unsigned)p.W);
-                    a[4 * u + e] = ok ? v[e] : 0.f;
-                }
-            }
-            // Pixels of the first image whose patch has padding on its left and holds input row 0: the
-            // 16-byte load of that row would begin before the tensor (a negative offset, which the range
-            // check rejects as a whole, in-range elements included).  Those few pixels take 4-byte loads.
-            if (live && b == 0 && h0 <= 0 && w0 < 0)
-            {
-#pragma unroll
-                for (int q = 0; q < TF_KH; ++q)
-                {
-                    const int kq = half * TF_KH + q;
-                    const int di = kq >> 4, t = kq & 15;
-                    const int dj = (int)p.fd_C.div((uint32_t)t);
-                    const bool ok = (int)(di < p.kh) & (int)(t < p.row) & (int)((unsigned)(h0 + di) < (unsigned)p.H) &
-                                    (int)((unsigned)(w0 + dj) < (unsigned)p.W);
-                    const int off = ok ? base + (di * p.W * p.C + t) * 4 : (int)0x80000000u;
-                    a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
-                }
+                const bool row_ok = (unsigned)(px.h0 + chunk_di[u]) < (unsigned)p.H;
+                const int off = row_ok ? base + chunk_off[u] : FAR;
+                raw[u] = __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(xr, off, 0, 0));
             }
         }
         else
@@ -273,39 +272,98 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
                 uint32_t di, t, dj, c;
                 p.fd_row.divmod(k, di, t);
                 p.fd_C.divmod(t, dj, c);
-                const bool ok = (int)live & (int)(k < p.K) & (int)((unsigned)(h0 + (int)di) < (unsigned)p.H) &
-                                (int)((unsigned)(w0 + (int)dj) < (unsigned)p.W);
-                const int off = ok ? base + ((int)di * p.W * p.C + (int)t) * 4 : (int)0x80000000u;
+                const bool ok = (int)px.live & (int)(k < p.K) & (int)((unsigned)(px.h0 + (int)di) < (unsigned)p.H) &
+                                (int)((unsigned)(px.w0 + (int)dj) < (unsigned)p.W);
+                const int off = ok ? px.base + ((int)di * p.W * p.C + (int)t) * 4 : (int)0x80000000u;
                 a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
             }
         }
-        {
-            // all of a thread's filter loads in flight together (out-of-range elements read element 0 and
-            // are replaced by zero: no branch around a load)
-            constexpr int PER_THREAD = 2 * TF_KH * 32 * TF_NB / 256;
-            float v[PER_THREAD];
+    };
+    auto finish = [&](const Pixel& px, const f32x4v (&raw)[TF_KH / 4], float (&a)[TF_KH]) {
+        if (!ROWS)
+            return;
+        // Element q of the lane is column t = (q + 8*half) mod 16 of its filter row; the columns that
+        // meet the image are tlo <= t < thi.  As a 16-bit mask rotated by the lane's 8*half, the bit
+        // of element q is bit q mod 16 -- a compile-time position: two ALU operations per element, no
+        // branches, and a NaN in a dropped element does not propagate (bitwise and).
+        const int tlo = max(0, -px.w0) * p.C, thi = min(p.row, (p.W - px.w0) * p.C);
+        uint32_t cols = thi > tlo ? ((1u << thi) - 1u) & ~((1u << tlo) - 1u) : 0u;
+        cols = half ? ((cols >> 8) | (cols << 8)) & 0xffffu : cols;
 #pragma unroll
-            for (int u = 0; u < PER_THREAD; ++u)
+        for (int u = 0; u < TF_KH / 4; ++u)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
             {
-                const int e = threadIdx.x + u * 256;
-                int k = e / (32 * TF_NB);
-                const int n = e - k * (32 * TF_NB);
-                bool ok = k < p.K && n < p.O;
-                if (ROWS)
-                {
-                    // k' = di*16 + t  ->  element (di*row + t) of the filter
-                    const int di = k >> 4, t = k & 15;
-                    ok = di < p.kh && t < p.row && n < p.O;
-                    k = di * p.row + t;
-                }
-                const float w = p.k[ok ? (size_t)k * p.O + n : 0];
-                v[u] = ok ? w : 0.f;
+                const int q = 4 * u + e;
+                const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)cols, q & 15, 1);   // 0 or all ones
+                const float v = raw[u][e];   // (a copy: bit_cast of a vector-element lvalue reads element 0)
+                a[q] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) & keep);
             }
+        if (px.corner)
+        {
 #pragma unroll
-            for (int u = 0; u < PER_THREAD; ++u)
-                filt[threadIdx.x + u * 256] = v[u];
+            for (int q = 0; q < TF_KH; ++q)
+            {
+                const int kq = half * TF_KH + q;
+                const int di = kq >> 4, t = kq & 15;
+                const int dj = (int)p.fd_C.div((uint32_t)t);
+                const bool ok = (int)(di < p.kh) & (int)(t < p.row) & (int)((unsigned)(px.h0 + di) < (unsigned)p.H) &
+                                (int)((unsigned)(px.w0 + dj) < (unsigned)p.W);
+                const int off = ok ? px.base + (di * p.W * p.C + t) * 4 : (int)0x80000000u;
+                a[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, off, 0, 0));
+            }
         }
-        __syncthreads();
+    };
+
+    // The wavefront's tiles: wave w of workgroup g takes tiles g*4 + w, + 4*gridDim.x, ...  The patch
+    // loads of the first are issued before the filter is staged, so that the two round trips to memory
+    // overlap; inside the loop the loads of the NEXT tile are issued before the MFMAs of the current
+    // one, so that a wavefront always has a tile's loads in flight while it multiplies and stores.
+    const int stride = (int)gridDim.x * 4;
+    int tile = (int)blockIdx.x * 4 + wave;
+    float a[TF_KH];
+    f32x4v raw[TF_KH / 4];
+    Pixel px = pixel_of(tile);
+    issue(px, raw, a);
+    {
+        // all of a thread's filter loads in flight together (out-of-range elements read element 0 and
+        // are replaced by zero: no branch around a load)
+        constexpr int PER_THREAD = 2 * TF_KH * 32 * TF_NB / 256;
+        float v[PER_THREAD];
+#pragma unroll
+        for (int u = 0; u < PER_THREAD; ++u)
+        {
+            const int e = threadIdx.x + u * 256;
+            int k = e / (32 * TF_NB);
+            const int n = e - k * (32 * TF_NB);
+            bool ok = k < p.K && n < p.O;
+            if (ROWS)
+            {
+                // k' = di*16 + t  ->  element (di*row + t) of the filter
+                const int di = k >> 4, t = k & 15;
+                ok = di < p.kh && t < p.row && n < p.O;
+                k = di * p.row + t;
+            }
+            const float w = p.k[ok ? (size_t)k * p.O + n : 0];
+            v[u] = ok ? w : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < PER_THREAD; ++u)
+            filt[threadIdx.x + u * 256] = v[u];
+    }
+    if (threadIdx.x < 32 * TF_NB)
+        lbias[threadIdx.x] = (p.bias && (int)threadIdx.x < p.O) ? p.bias[threadIdx.x] : 0.f;
+    __syncthreads();
+
+    for (; tile < p.tiles; tile += stride)
+    {
+        // (the filter values are read from LDS in every round: kept in registers across the loop they
+        // would take 160 of them and halve the wavefronts a SIMD holds)
+        asm volatile("" ::: "memory");
+        finish(px, raw, a);
+        px = pixel_of(tile + stride);
+        float a_next[TF_KH];
+        issue(px, raw, a_next);
         f32x16 acc[TF_NB];
 #pragma unroll
         for (int nb = 0; nb < TF_NB; ++nb)
@@ -319,7 +377,8 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
                 acc[nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bw[q * (32 * TF_NB) + nb * 32], a[q], acc[nb], 0, 0, 0);
 
         // register r of lane (m, h) holds channel 32*nb + 8*(r/4) + 4*h + r%4 of pixel m
-        if (live)
+        const int pix = tile * 32 + l32;
+        if (pix < p.pixels)
         {
             float* dst = p.y + (size_t)pix * p.O;
 #pragma unroll
@@ -330,19 +389,23 @@ __global__ __launch_bounds__(256) void fwd_thin(const ThinFwdParams p)
                     const int n = nb * 32 + 8 * g + 4 * half;
                     if (n >= p.O)
                         continue;
+                    const float4 bb = *reinterpret_cast<const float4*>(lbias + n);
                     float4 v = make_float4(acc[nb][4 * g], acc[nb][4 * g + 1], acc[nb][4 * g + 2], acc[nb][4 * g + 3]);
-                    if (p.bias)
-                    {
-                        const float4 bb = *reinterpret_cast<const float4*>(p.bias + n);
-                        v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
-                    }
+                    v.x += bb.x; v.y += bb.y; v.z += bb.z; v.w += bb.w;
                     v.x = act_apply(v.x, p.act, p.alpha); v.y = act_apply(v.y, p.act, p.alpha);
                     v.z = act_apply(v.z, p.act, p.alpha); v.w = act_apply(v.w, p.act, p.alpha);
                     *reinterpret_cast<float4*>(dst + n) = v;
                 }
         }
+        if (!ROWS)
+        {
+#pragma unroll
+            for (int q = 0; q < TF_KH; ++q)
+                a[q] = a_next[q];
+        }
     }
 }
+
 
 
 // ---- filter gradient of a thin input ------------------------------------------------------------
@@ -576,9 +639,16 @@ int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W,
     p.pixels = N * Ho * Wo;
     p.x_bytes = (uint32_t)x_bytes;
     p.fd_HoWo = FastDiv((uint32_t)Ho * Wo); p.fd_Wo = FastDiv(Wo); p.fd_row = FastDiv(kw * C); p.fd_C = FastDiv(C);
-    const long blocks = ((long)(p.pixels + 31) / 32 + 3) / 4;   // four wavefronts, one 32-pixel tile each
-    if (blocks > 0x7fffffffL)
+    // four wavefronts per workgroup, each walking over 32-pixel tiles; at most two workgroups per compute
+    // unit (two wavefronts per SIMD: one multiplies while the other waits for its loads or drains its stores)
+    const long tiles = ((long)p.pixels + 31) / 32;
+    if (tiles > 0x3fffffffL)
         return 1;
+    p.tiles = (int)tiles;
+    long blocks = (tiles + 3) / 4;
+    const long resident = 2L * num_cus();
+    if (blocks > resident)
+        blocks = resident;
     const int prof = prof_begin("fwd_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
     if (kw * C <= 16 && kh * 16 <= 2 * TF_KH)
         hipLaunchKernelGGL(fwd_thin<true>, dim3((unsigned)blocks), dim3(256), 0, st, p);
