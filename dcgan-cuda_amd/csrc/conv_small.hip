@@ -410,24 +410,33 @@ __global__ __launch_bounds__(256, 2) void fwd_thin(const ThinFwdParams p)
 
 // ---- filter gradient of a thin input ------------------------------------------------------------
 // dk[(di,dj,c), o] = sum over pixels of x[b, i*sh+di-pt, j*sw+dj-pl, c] * dy[b,i,j,o] for a filter
-// with at most 96 elements per output channel and at most 64 output channels (the discriminator's
+// with at most 80 elements per output channel and at most 64 output channels (the discriminator's
 // first layer: 75 x 64).  As an implicit GEMM it is a 75-row product whose "im2col" operand has to
 // be gathered element by element (3 channels); here a wavefront takes segments of 16 neighbouring
 // output pixels of one image row and stages, per segment, the kh input rows they touch and their
 // 16 dy pixels in LDS.  Element ((di, dj, c), j) of the gathered operand is then
 //     patch[di][(dj*C + c) + j*sw*C]
 // -- a strided view of the staged rows, read straight into the MFMA registers with no gather at all.
-// The four wavefronts of a workgroup work on different segments and add their accumulators through
-// LDS in wavefront order; each workgroup writes one slice of partial sums, which the caller adds
-// up (fixed order, so the result is repeatable to the bit).
-typedef float dt_f32x16 __attribute__((ext_vector_type(16)));
+// The result is tiled 5 x 4 by 16x16x4 MFMAs (80 x 64: 6 % padding for the 75-row filter, where 32-wide
+// tiles would waste 22 %).  Each wavefront has staging memory of its own and LDS operations of one
+// wavefront execute in order, so the segment loop needs no barrier: a wavefront writes segment s+1 over
+// segment s as soon as its own fragment reads of s are issued, and the global loads of the segment after
+// are in flight meanwhile.  Two wavefronts share a SIMD.  The eight wavefronts of a workgroup add their
+// accumulators through LDS in wavefront order; each workgroup writes one slice of partial sums, which
+// the caller adds up (fixed order, so the result is repeatable to the bit).
+typedef float dt_f32x4 __attribute__((ext_vector_type(4)));
 constexpr int DT_SEG = 16;                    // output pixels per segment
 constexpr int DT_XMAX = 640;                  // floats of one staged input patch (kh rows)
-constexpr int DT_OMAX = 64;                   // output channels, and the LDS stride of a dy pixel
+constexpr int DT_OMAX = 64;                   // output channels
+constexpr int DT_OSTRIDE = 80;                // LDS stride of a dy pixel: the 4 pixels of a fragment read fall into disjoint banks
 constexpr int DT_XPL = DT_XMAX / 64;          // patch elements a lane loads
-constexpr int DT_WAVE_LDS = DT_XMAX + DT_SEG * DT_OMAX + 64;   // floats per wavefront (the last 64: zeros)
-constexpr int DT_MT = 3, DT_NT = 2;           // 32x32 MFMA tiles of the result
-static_assert(4 * DT_WAVE_LDS >= DT_MT * 32 * DT_OMAX, "the accumulators of a workgroup are added in its staging memory");
+constexpr int DT_WAVES = 8;
+constexpr int DT_MT = 5, DT_NT = 4;           // 16x16 MFMA tiles of the result
+// floats per wavefront (the last 64: zeros); eight of them also hold the four regions in which the
+// accumulators of a workgroup are added up
+constexpr int DT_WAVE_LDS = 4 * DT_MT * 16 * DT_OMAX / DT_WAVES;
+constexpr int DT_DUMP = DT_XMAX + DT_SEG * DT_OSTRIDE + 64;   // 64 + 256 floats that nothing reads
+static_assert(DT_WAVE_LDS >= DT_DUMP + 64 + 256, "staging memory of a wavefront");
 
 struct ThinDkParams
 {
@@ -442,18 +451,20 @@ struct ThinDkParams
     int rsw;              // floats of a staged input row: (DT_SEG - 1) * sw * C + kw * C
     int rs;               // its LDS stride (bank-conflict-free fragment reads)
     int segs_per_row, total_segs, segs_per_wave;
+    uint32_t x_bytes, dy_bytes;
     FastDiv fd_segs_per_row, fd_Ho, fd_rsw, fd_row, fd_O4;
 };
 
-__global__ __launch_bounds__(256) void dk_thin(const ThinDkParams p)
+__global__ __launch_bounds__(64 * DT_WAVES, 2) void dk_thin(const ThinDkParams p)
 {
-    __shared__ __attribute__((aligned(16))) float lds[4 * DT_WAVE_LDS];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ __attribute__((aligned(16))) float lds[DT_WAVES * DT_WAVE_LDS];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // (scalar: segment arithmetic runs on the scalar unit)
     float* lx = lds + wave * DT_WAVE_LDS;
     float* ld = lx + DT_XMAX;
-    float* lzero = ld + DT_SEG * DT_OMAX;
+    float* lzero = ld + DT_SEG * DT_OSTRIDE;
     lzero[lane] = 0.f;
-    const int s_begin = ((int)blockIdx.x * 4 + wave) * p.segs_per_wave;
+    const int s_begin = ((int)blockIdx.x * DT_WAVES + wave) * p.segs_per_wave;
     const int s_end = min(p.total_segs, s_begin + p.segs_per_wave);
 
     // patch elements of this lane: e = lane + 64 q -> (row r, column col) of the staged rows
@@ -477,142 +488,190 @@ __global__ __launch_bounds__(256) void dk_thin(const ThinDkParams p)
         d_pix[q] = (int)pix < DT_SEG ? (int)pix : (1 << 28);
         d_o4[q] = (int)o4;
     }
-    // MFMA fragments: A[m = (di, dj*C + c)][k = pixel], B[k = pixel][n = o]; lanes 32-63 hold the second pixel
-    const int l32 = lane & 31, half = lane >> 5;
+    // MFMA fragments (16x16x4): A[m = (di, dj*C + c)][k = pixel], B[k = pixel][n = o]; lane (l16, kq)
+    // supplies row / column l16 for pixel kq of each group of four
+    const int l16 = lane & 15, kq = lane >> 4;
     // (rows and columns past the result's extents read a zero word, with a step of zero)
     int a_ptr[DT_MT], b_ptr[DT_NT];   // offsets into this wavefront's LDS
-    int a_step[DT_MT], b_step[DT_NT];
-    const int zero_at = DT_XMAX + DT_SEG * DT_OMAX + lane;
+    int a_step[DT_MT], b_step[DT_NT]; // per group of four pixels
+    const int zero_at = DT_XMAX + DT_SEG * DT_OSTRIDE + lane;
 #pragma unroll
     for (int mt = 0; mt < DT_MT; ++mt)
     {
-        const int m = mt * 32 + l32;
+        const int m = mt * 16 + l16;
         uint32_t di, mp;
         p.fd_row.divmod(m, di, mp);
-        a_ptr[mt] = m < p.M ? (int)di * p.rs + (int)mp + half * p.sw * p.C : zero_at;
-        a_step[mt] = m < p.M ? p.sw * p.C : 0;
+        a_ptr[mt] = m < p.M ? (int)di * p.rs + (int)mp + kq * p.sw * p.C : zero_at;
+        a_step[mt] = m < p.M ? 4 * p.sw * p.C : 0;
     }
 #pragma unroll
     for (int nt = 0; nt < DT_NT; ++nt)
     {
-        const int n = nt * 32 + l32;
-        b_ptr[nt] = n < p.O ? DT_XMAX + half * DT_OMAX + n : zero_at;
-        b_step[nt] = n < p.O ? DT_OMAX : 0;
+        const int n = nt * 16 + l16;
+        b_ptr[nt] = n < p.O ? DT_XMAX + kq * DT_OSTRIDE + n : zero_at;
+        b_step[nt] = n < p.O ? 4 * DT_OSTRIDE : 0;
     }
-    dt_f32x16 acc[DT_MT][DT_NT];
+    dt_f32x4 acc[DT_MT][DT_NT];
 #pragma unroll
     for (int mt = 0; mt < DT_MT; ++mt)
 #pragma unroll
         for (int nt = 0; nt < DT_NT; ++nt)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
+            for (int r = 0; r < 4; ++r)
                 acc[mt][nt][r] = 0.f;
 
-    float xv[DT_XPL];
-    float4 dv[4];
-    auto load = [&](int s) {
+    // two register sets: the loads of a segment are issued two segments ahead of its use
+    float xv0[DT_XPL], xv1[DT_XPL];
+    float4 dv0[4], dv1[4];
+    // Loads go through buffer descriptors: an element that does not exist (outside the image, past the
+    // row's end, a segment past the wavefront's last) gets an out-of-range offset and reads as zero, so
+    // that the loop body is one basic block and the loads of a segment are issued back to back.
+    const __amdgpu_buffer_rsrc_t xr1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xr2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x2 ? p.x2 : p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t dr1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t dr2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.dy2 ? p.dy2 : p.dy), 0, (int)p.dy_bytes, 0x00020000);
+    constexpr uint32_t FAR = 0xffffff00u;     // beyond any tensor the kernel takes (below 4 GiB - 256 bytes)
+    auto load = [&](int s, float (&xv)[DT_XPL], float4 (&dv)[4]) {
+        const bool live = s < s_end;
         uint32_t bi, js, b, i;
-        p.fd_segs_per_row.divmod(s, bi, js);
+        p.fd_segs_per_row.divmod(live ? s : 0, bi, js);
         p.fd_Ho.divmod(bi, b, i);
         const int j0 = (int)js * DT_SEG;
         const int ih0 = (int)i * p.sh - p.pt;
         const int g0 = (j0 * p.sw - p.pl) * p.C;      // first staged column, in floats from the row start
         const bool second = (int)b >= p.N;       // only with a second pair of operands
         b -= second ? (uint32_t)p.N : 0u;
-        const float* xrow = (second ? p.x2 : p.x) + ((size_t)b * p.H) * p.W * p.C;
-        const ptrdiff_t base = (ptrdiff_t)ih0 * p.W * p.C + g0;
-        // every lane loads (from the start of the image where its element does not exist) and the value
-        // is dropped afterwards, so that the loads are issued back to back
+        const __amdgpu_buffer_rsrc_t xr = second ? xr2 : xr1;
+        const __amdgpu_buffer_rsrc_t dr = second ? dr2 : dr1;
+        // byte offset of the staged patch's origin, modulo 2^32 (exact for every element that exists:
+        // the tensors are below 4 GiB)
+        const uint32_t origin = ((b * (uint32_t)p.H + (uint32_t)ih0) * (uint32_t)(p.W * p.C) + (uint32_t)g0) * 4u;
+        const uint32_t row_bytes = (uint32_t)(p.W * p.C) * 4u;
 #pragma unroll
         for (int q = 0; q < DT_XPL; ++q)
         {
             const int r = x_rc[q] >> 16, col = x_rc[q] & 0xffff;
             const int ih = ih0 + r, g = g0 + col;
-            const bool ok = (unsigned)ih < (unsigned)p.H && (unsigned)g < (unsigned)(p.W * p.C);
-            const float v = xrow[ok ? base + r * p.W * p.C + col : 0];
-            xv[q] = ok ? v : 0.f;
+            const bool ok = (int)live & (int)((unsigned)ih < (unsigned)p.H) & (int)((unsigned)g < (unsigned)(p.W * p.C));
+            const uint32_t off = ok ? origin + (uint32_t)r * row_bytes + (uint32_t)col * 4u : FAR;
+            xv[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)off, 0, 0));
         }
-        const float* drow = (second ? p.dy2 : p.dy) + (((size_t)b * p.Ho + i) * p.Wo + j0) * p.O;
+        const uint32_t drow = ((b * (uint32_t)p.Ho + i) * (uint32_t)p.Wo + (uint32_t)j0) * (uint32_t)p.O * 4u;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
         {
-            const bool ok = d_pix[q] < DT_SEG && j0 + d_pix[q] < p.Wo;
-            const float4 t = *reinterpret_cast<const float4*>(drow + (ok ? d_pix[q] * p.O + d_o4[q] * 4 : 0));
-            dv[q] = ok ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+            const bool ok = (int)live & (int)(d_pix[q] < DT_SEG) & (int)(j0 + d_pix[q] < p.Wo);
+            const uint32_t off = ok ? drow + ((uint32_t)d_pix[q] * (uint32_t)p.O + (uint32_t)d_o4[q] * 4u) * 4u : FAR;
+            const dt_f32x4 t = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(dr, (int)off, 0, 0));
+            dv[q] = make_float4(t[0], t[1], t[2], t[3]);
         }
     };
-    auto stash = [&]() {
+    // where this lane's elements go in the staging memory (an element that does not exist goes to a
+    // dump word of the lane's own: no branch around a write)
+    int x_lds[DT_XPL], d_lds[4];
+#pragma unroll
+    for (int q = 0; q < DT_XPL; ++q)
+        x_lds[q] = (x_rc[q] >> 16) != 0x7fff ? (x_rc[q] >> 16) * p.rs + (x_rc[q] & 0xffff) : DT_DUMP + lane;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        d_lds[q] = d_pix[q] < DT_SEG ? DT_XMAX + d_pix[q] * DT_OSTRIDE + d_o4[q] * 4 : DT_DUMP + 64 + 4 * lane;
+    auto stash = [&](const float (&xv)[DT_XPL], const float4 (&dv)[4]) {
 #pragma unroll
         for (int q = 0; q < DT_XPL; ++q)
-            if ((x_rc[q] >> 16) != 0x7fff)
-                lx[(x_rc[q] >> 16) * p.rs + (x_rc[q] & 0xffff)] = xv[q];
+            lx[x_lds[q]] = xv[q];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            if (d_pix[q] < DT_SEG)
-                *reinterpret_cast<float4*>(ld + d_pix[q] * DT_OMAX + d_o4[q] * 4) = dv[q];
+            *reinterpret_cast<float4*>(lx + d_lds[q]) = dv[q];
     };
 
-    if (s_begin < s_end)
-        load(s_begin);
-    for (int it = 0; it < p.segs_per_wave; ++it)   // the same trip count in every wavefront: barriers inside
-    {
-        const int s = s_begin + it;
-        __syncthreads();
-        if (s < s_end)
-            stash();
-        __syncthreads();
-        if (s + 1 < s_end)
-            load(s + 1);
-        if (s < s_end)
-        {
-            // fully unrolled: the LDS reads of all eight steps are issued ahead of the MFMAs (340 registers,
-            // one wavefront per SIMD -- which is all the launch has anyway)
+    auto multiply = [&]() {
+        // the fragments of a group of four pixels are read while the MFMAs of the group before run
+        float a[2][DT_MT], b[2][DT_NT];
 #pragma unroll
-            for (int jj = 0; jj < DT_SEG; jj += 2)
+        for (int mt = 0; mt < DT_MT; ++mt)
+            a[0][mt] = lx[a_ptr[mt]];
+#pragma unroll
+        for (int nt = 0; nt < DT_NT; ++nt)
+            b[0][nt] = lx[b_ptr[nt]];
+#pragma unroll
+        for (int jj = 0; jj < DT_SEG / 4; ++jj)
+        {
+            const int cur = jj & 1, nxt = cur ^ 1;
+            if (jj + 1 < DT_SEG / 4)
             {
-                float a[DT_MT], b[DT_NT];
 #pragma unroll
                 for (int mt = 0; mt < DT_MT; ++mt)
-                    a[mt] = lx[a_ptr[mt] + jj * a_step[mt]];
+                    a[nxt][mt] = lx[a_ptr[mt] + (jj + 1) * a_step[mt]];
 #pragma unroll
                 for (int nt = 0; nt < DT_NT; ++nt)
-                    b[nt] = lx[b_ptr[nt] + jj * b_step[nt]];
-#pragma unroll
-                for (int mt = 0; mt < DT_MT; ++mt)
-#pragma unroll
-                    for (int nt = 0; nt < DT_NT; ++nt)
-                        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mt], b[nt], acc[mt][nt], 0, 0, 0);
+                    b[nxt][nt] = lx[b_ptr[nt] + (jj + 1) * b_step[nt]];
             }
+#pragma unroll
+            for (int mt = 0; mt < DT_MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < DT_NT; ++nt)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[cur][mt], b[cur][nt], acc[mt][nt], 0, 0, 0);
         }
+    };
+    // LDS operations of one wavefront execute in program order: the writes of a segment come after the
+    // fragment reads of the segment before, the reads after them see the new segment.  The fences keep
+    // the compiler from moving them across each other; no instruction results from them.
+    auto step = [&](int s, float (&xv)[DT_XPL], float4 (&dv)[4]) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        stash(xv, dv);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        load(s + 2, xv, dv);
+        multiply();
+    };
+
+    // (an odd last segment runs as a segment of zeros: every load of it is out of range)
+    load(s_begin, xv0, dv0);
+    load(s_begin + 1, xv1, dv1);
+    for (int s = s_begin; s < s_end; s += 2)
+    {
+        step(s, xv0, dv0);
+        step(s + 1, xv1, dv1);
     }
 
-    // add the four accumulators in wavefront order; register r of lane l holds element
-    // (m = 8 * (r / 4) + 4 * (l / 32) + r % 4, n = l % 32) of its 32x32 tile
+    // Add the eight accumulators in a fixed order: wavefronts 0-3 put theirs into four regions of the
+    // staging memory, wavefronts 4-7 add theirs on top (region w - 4), then every thread adds the four
+    // regions of its elements in region order and writes them to the workgroup's slice.  Register r of
+    // lane (l16, kq) holds element (m = 4 * kq + r, n = l16) of its 16x16 tile.
+    constexpr int REGION = DT_MT * 16 * DT_OMAX;
     __syncthreads();
-    for (int w = 0; w < 4; ++w)
+    for (int round = 0; round < 2; ++round)
     {
-        if (wave == w)
+        if ((wave >> 2) == round)
         {
+            float* reg = lds + (wave & 3) * REGION;
 #pragma unroll
             for (int mt = 0; mt < DT_MT; ++mt)
 #pragma unroll
                 for (int nt = 0; nt < DT_NT; ++nt)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
+                    for (int r = 0; r < 4; ++r)
                     {
-                        const int m = mt * 32 + 8 * (r / 4) + 4 * half + r % 4, n = nt * 32 + l32;
-                        float* dst = lds + m * DT_OMAX + n;
-                        *dst = w == 0 ? acc[mt][nt][r] : *dst + acc[mt][nt][r];
+                        float* dst = reg + (mt * 16 + 4 * kq + r) * DT_OMAX + nt * 16 + l16;
+                        *dst = round == 0 ? acc[mt][nt][r] : *dst + acc[mt][nt][r];
                     }
         }
         __syncthreads();
     }
     const int total = p.M * p.O;
     float* out = p.part + (size_t)blockIdx.x * total;
-    for (int idx = threadIdx.x * 4; idx < total; idx += 256 * 4)
+    for (int idx = threadIdx.x * 4; idx < total; idx += 64 * DT_WAVES * 4)
     {
         const int m = idx / p.O, n = idx - m * p.O;   // O is a multiple of 4: a quad stays in its row
-        *reinterpret_cast<float4*>(out + idx) = *reinterpret_cast<const float4*>(lds + m * DT_OMAX + n);
+        const float* src = lds + m * DT_OMAX + n;
+        float4 v = *reinterpret_cast<const float4*>(src);
+#pragma unroll
+        for (int g = 1; g < 4; ++g)
+        {
+            const float4 t = *reinterpret_cast<const float4*>(src + g * REGION);
+            v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+        }
+        *reinterpret_cast<float4*>(out + idx) = v;
     }
 }
 
@@ -724,8 +783,10 @@ bool dk_thin_takes(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, in
     const int M = kh * kw * C, row = kw * C;
     const int rsw = (DT_SEG - 1) * sw * C + row;
     const int rs = rsw + ((row - rsw) % 32 + 32) % 32;
-    return !(M > DT_MT * 32 || O > DT_OMAX || O % 4 != 0 || kh * rs > DT_XMAX || kh * rsw > 64 * DT_XPL ||
-             (long)N * Ho * Wo < 2048 || (double)N * H * W * C >= 2147483647.0);
+    // (both operand tensors below 4 GiB - 256 bytes: 32-bit byte offsets into buffer descriptors)
+    return !(M > DT_MT * 16 || O > DT_OMAX || O % 4 != 0 || kh * rs > DT_XMAX || kh * rsw > 64 * DT_XPL ||
+             (long)N * Ho * Wo < 2048 || (double)N * H * W * C * 4.0 >= 4294967040.0 ||
+             (double)N * Ho * Wo * O * 4.0 >= 4294967040.0);
 }
 
 // x2 / dy2: a second pair of operands whose filter gradient is added to the first's (both null: one pair).
@@ -744,17 +805,18 @@ int conv_dk_thin(const float* x, const float* dy, const float* x2, const float* 
     p.N = N; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.O = O; p.kh = kh; p.kw = kw;
     p.sh = sh; p.sw = sw; p.pt = pt; p.pl = pl;
     p.M = M; p.row = row; p.rsw = rsw; p.rs = rs;
+    p.x_bytes = (uint32_t)((size_t)N * H * W * C * 4); p.dy_bytes = (uint32_t)((size_t)N * Ho * Wo * O * 4);
     p.segs_per_row = (Wo + DT_SEG - 1) / DT_SEG;
     const long total = (long)images * Ho * p.segs_per_row;
     if (total > 0x7fffffffL)
         return 1;
     p.total_segs = (int)total;
-    // one workgroup per compute unit (two measured the same: the kernel is bound by the latency of a
-    // segment's load - stage - multiply chain, not by throughput), at least two segments per wavefront
+    // one workgroup of eight wavefronts per compute unit (two wavefronts per SIMD: one multiplies while
+    // the other stages its next segment), at least two segments per wavefront
     long wgs = 1L * num_cus();
-    long per_wave = (total + wgs * 4 - 1) / (wgs * 4);
+    long per_wave = (total + wgs * DT_WAVES - 1) / (wgs * DT_WAVES);
     if (per_wave < 2) per_wave = 2;
-    wgs = (total + per_wave * 4 - 1) / (per_wave * 4);
+    wgs = (total + per_wave * DT_WAVES - 1) / (per_wave * DT_WAVES);
     p.segs_per_wave = (int)per_wave;
     p.fd_segs_per_row = FastDiv(p.segs_per_row); p.fd_Ho = FastDiv(Ho); p.fd_rsw = FastDiv(rsw);
     p.fd_row = FastDiv(row); p.fd_O4 = FastDiv(O / 4);
@@ -762,7 +824,7 @@ int conv_dk_thin(const float* x, const float* dy, const float* x2, const float* 
     DH_TRY(workspace((size_t)wgs * M * O * sizeof(float), &ws, st));
     p.part = static_cast<float*>(ws);
     const int prof = prof_begin("dk_thin", 2.0 * images * Ho * Wo * O * kh * kw * C, st);
-    hipLaunchKernelGGL(dk_thin, dim3((unsigned)wgs), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(dk_thin, dim3((unsigned)wgs), dim3(64 * DT_WAVES), 0, st, p);
     prof_end(prof, st);
     DH_LAUNCH_CHECK("dk_thin launch");
     *part = p.part;

@@ -59,7 +59,7 @@ int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int 
 int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
                   int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st);
 
-// Filter gradient of a thin input (at most 96 filter elements per output channel, at most 64 output
+// Filter gradient of a thin input (at most 80 filter elements per output channel, at most 64 output
 // channels): writes *splits slices of partial sums to the scratch arena and returns them in *part for
 // the caller to add up; same return convention.
 // x2 / dy2 (both null, or both set): a second pair of operands contracted into the same result.

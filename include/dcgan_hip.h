@@ -175,7 +175,7 @@ int dh_conv2d_dk(const float* x, const float* dy, float* dk,
  * contracts over -- the input's for fwd, dy's for dx -- by 16; 16-byte aligned tensors below 2 GiB)
  * and return DH_ENOTSUP otherwise; results agree with the single calls to rounding
  * (the contraction may be split differently).  dh_conv2d_dk_pair also takes the thin-input filter
- * gradient (at most 96 filter elements per output channel, at most 64 output channels: the image
+ * gradient (at most 80 filter elements per output channel, at most 64 output channels: the image
  * layer); dh_conv2d_dk_pair_supported tells a caller that plans its launches ahead whether a geometry
  * is one the paired filter gradient takes (1) or not (0), 16-byte aligned tensors assumed. */
 int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,
