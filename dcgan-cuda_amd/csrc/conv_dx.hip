@@ -17,6 +17,10 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
     if (!dy || !k || !dx || (pair && (!dy2 || !dx2))) return fail(DH_EINVAL, "%s: null tensor", who);
     if (!pair && !g_force_generic)
     {
+        const int rc0 = conv_dx_col2im(dy, k, dx, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias, act, alpha,
+                                       as_stream(stream));
+        if (rc0 != 1)
+            return rc0;
         const int rc = conv_dx_few_channels(dy, k, dx, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias,
                                             act, alpha, as_stream(stream));
         if (rc != 1)

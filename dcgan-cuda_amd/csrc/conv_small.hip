@@ -675,6 +675,268 @@ __global__ __launch_bounds__(64 * DT_WAVES, 2) void dk_thin(const ThinDkParams p
     }
 }
 
+// ---- transposed convolution onto few channels as a product followed by in-register sums ----------
+// The generator's image layer, [N,32,32,64] -> [N,64,64,3] (5x5, stride 2), and the gradient of the
+// discriminator's first layer.  Written as dx[b, 2i+di-1, 2j+dj-1, c] += Z[(b,i,j), (di,dj,c)] with
+//     Z[pixel, (di,dj,c)] = sum_o dy[pixel, o] * k[(di,dj,c), o]
+// the arithmetic is ONE dense product, 75 x pixels x 64, with no product against an inserted zero and
+// no tap enumeration: it runs on the matrix cores (16x16x4 tiles), and what remains is to add up, for
+// every output element, the 4 to 9 entries of Z that land on it.
+//   * The filter is the MFMA's A operand, 80 values per lane for the whole kernel: tile dj holds, in
+//     row 3 di + c, the filter row (di, dj, c) (row 15 is zero).  A row of 32 dy pixels is the B operand
+//     of two tiles: tile t holds pixel 2 n + t in column n, lane (n, q) loading channels 16q .. 16q+15
+//     of its pixel straight from global memory into the registers the MFMAs consume.  A wavefront
+//     multiplies one dy row per step (160 MFMAs); the loads of the next row are issued before them.
+//   * ACROSS a row: the result lane (n, q) holds Z[pixel 2n+t][(di,c) = 4q+r][dj] in register r of
+//     accumulator (t, dj) -- all five dj of a pixel in ONE lane, and the neighbouring pixels 2n-1 and
+//     2n+2 one lane to the left and right.  The sums over dj for the output columns 4n .. 4n+3 are
+//     therefore register adds, three of them through a one-lane row shift (DPP): 28 adds give
+//     R[(di,c)][w], the row of Z summed over dj, 16 x 64 values, which the wavefront writes to a ring
+//     of three rows in LDS that only it reads (4 KB a row; LDS operations of one wavefront execute in
+//     order, so no barrier).
+//   * DOWN the rows: lane w then adds, for the row before, the two output rows it completes from R of
+//     three consecutive dy rows (5 reads per channel), applies bias and activation and stores them.
+//   * Eight wavefronts share a strip of rows of one image, each taking consecutive rows.  Wavefronts
+//     w and w + 4 run on one SIMD: their MFMA bursts alternate (timestamps show one burst of 160 at a
+//     time, 5440 cycles each, 200 to 600 cycles apart), and the sums and stores of one proceed while
+//     the other multiplies.  fp32 MFMAs and vector instructions share the SIMD's ALU here -- a loop
+//     of MFMAs and one of FMAs in two wavefronts of a SIMD take the sum of their times -- so every
+//     vector instruction saved is matrix time gained; that is why the sums run across lanes in
+//     registers instead of gathering from LDS.
+//   * The first and the last row of a wavefront also need R of the neighbouring wavefront's last and
+//     first row: those parts (9 x 64 values) are published in LDS, and after ONE barrier per strip
+//     every wavefront finishes its two edge rows.  Strips that are not whole images compute one row
+//     above and below what they own.
+// Takes 5x5 filters, stride 2, one pixel of padding before, at most 3 result channels, 64 dy channels,
+// dy rows of at most 32 pixels; other shapes keep dx_few_channels.
+// Reference counterpart: kernel_conv2d_transpose / kernel_conv2d_input_grad (src/gpu/conv2d.cu:70-117,
+// 167-212).
+constexpr int CT_PIX = 32;          // pixels of a dy row (two 16-pixel MFMA tiles)
+constexpr int CT_WAVES = 8;         // wavefronts per workgroup
+constexpr int CT_RING = 3;          // rows of R a wavefront keeps
+constexpr int CT_ROWF = 16 * 64;    // floats in a row of R: 16 (di,c) slots x 64 output columns
+constexpr int CT_KS = 16;           // MFMA steps: 64 dy channels, 4 per step
+
+struct Col2imParams
+{
+    const float* dy;
+    const float* k;
+    float* dx;
+    const float* bias;
+    int act;
+    float alpha;
+    int N, Ho, Wo, C, H, W;
+    int rows_per_strip, strips_per_image, strips;
+    uint32_t dy_bytes;
+};
+
+// value of lane n-1 (n+1) of the same 16-lane row, zero at the row's end
+__device__ __forceinline__ float ct_from_left(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float ct_from_right(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x101, 0xf, 0xf, true));
+}
+
+__global__ __launch_bounds__(64 * CT_WAVES, 2) void dx_col2im(const Col2imParams p)
+{
+    __shared__ __attribute__((aligned(16))) float ring[CT_WAVES][CT_RING][CT_ROWF];
+    __shared__ float xfirst[CT_WAVES][3 * 64];   // R[(0,c)] of a wavefront's first row
+    __shared__ float xlast[CT_WAVES][6 * 64];    // R[(3,c)], R[(4,c)] of its last row
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l16 = lane & 15, kq = lane >> 4;
+
+    // the filter as MFMA operand A[m = (di,c)][k = o] of tile dj: lane (m, q) holds o = 16q .. 16q+15
+    float aq[5][CT_KS];
+    {
+        const int di = l16 / 3, c = l16 - 3 * di;
+        const bool ok = l16 < 15 && c < p.C;
+#pragma unroll
+        for (int dj = 0; dj < 5; ++dj)
+        {
+            const float* src = p.k + (size_t)(ok ? (di * 5 + dj) * p.C + c : 0) * 64 + kq * 16;
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+            {
+                const float4 v = *reinterpret_cast<const float4*>(src + 4 * g);
+                aq[dj][4 * g + 0] = ok ? v.x : 0.f; aq[dj][4 * g + 1] = ok ? v.y : 0.f;
+                aq[dj][4 * g + 2] = ok ? v.z : 0.f; aq[dj][4 * g + 3] = ok ? v.w : 0.f;
+            }
+        }
+    }
+    const float bias_c[3] = {p.bias && p.C > 0 ? p.bias[0] : 0.f, p.bias && p.C > 1 ? p.bias[1] : 0.f,
+                             p.bias && p.C > 2 ? p.bias[2] : 0.f};
+    const __amdgpu_buffer_rsrc_t dr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
+    constexpr uint32_t FAR = 0xffffff00u;
+    float* const my_ring = &ring[wave][0][0];
+
+    for (int strip = blockIdx.x; strip < p.strips; strip += gridDim.x)
+    {
+        const int b = strip / p.strips_per_image;
+        const int own0 = (strip - b * p.strips_per_image) * p.rows_per_strip;
+        const int own1 = min(p.Ho, own0 + p.rows_per_strip);
+        const int c0 = max(0, own0 - 1), c1 = min(p.Ho, own1 + 1);      // rows of Z the strip computes
+        const int row_a = c0 + wave * (c1 - c0) / CT_WAVES, row_b = c0 + (wave + 1) * (c1 - c0) / CT_WAVES;
+
+        // dy[b, i, 2 n + t, 16 q ..] for both tiles of row i: zeros past the wavefront's rows or the row's end
+        auto issue = [&](int i, dt_f32x4 (&raw)[2][4]) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+            {
+                const int jpix = 2 * l16 + t;
+                const bool ok = (int)(i < row_b) & (int)(jpix < p.Wo);
+                const uint32_t off = ((((uint32_t)b * p.Ho + (uint32_t)i) * p.Wo + (uint32_t)jpix) * 64u + (uint32_t)kq * 16u) * 4u;
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    raw[t][g] = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(dr, (int)(ok ? off + 16u * g : FAR), 0, 0));
+            }
+        };
+        // the parts of output rows 2i and 2i+1, column `lane`, that come from R of row i / i-1 / i+1
+        auto add_mid = [&](const float* r, float (&o)[6]) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) { o[c] += r[(3 + c) * 64 + lane]; o[3 + c] += r[(6 + c) * 64 + lane]; }
+        };
+        auto add_up = [&](const float* r3, const float* r4, float (&o)[6]) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) { o[c] += r3[c * 64 + lane]; o[3 + c] += r4[c * 64 + lane]; }
+        };
+        auto add_down = [&](const float* r0, float (&o)[6]) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) o[3 + c] += r0[c * 64 + lane];
+        };
+        auto store = [&](int i, const float (&o)[6]) {
+            if (i < own0 || i >= own1 || lane >= p.W)
+                return;
+            float* dst = p.dx + (((size_t)b * p.H + 2 * i) * p.W + lane) * p.C;
+#pragma unroll
+            for (int c = 0; c < 3; ++c)
+                if (c < p.C)
+                {
+                    dst[c] = act_apply(o[c] + bias_c[c], p.act, p.alpha);
+                    dst[(size_t)p.W * p.C + c] = act_apply(o[3 + c] + bias_c[c], p.act, p.alpha);
+                }
+        };
+
+        float edge_first[6], edge_last[6];      // the wavefront's first and last row, still without the neighbours' parts
+        dt_f32x4 b_cur[2][4], b_next[2][4];
+        if (row_a < row_b)
+            issue(row_a, b_cur);
+        for (int i = row_a; i < row_b; ++i)
+        {
+            issue(i + 1, b_next);
+            dt_f32x4 acc[2][5];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int dj = 0; dj < 5; ++dj)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        acc[t][dj][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < CT_KS; ++s)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                {
+                    const float bv = b_cur[t][s >> 2][s & 3];
+#pragma unroll
+                    for (int dj = 0; dj < 5; ++dj)
+                        acc[t][dj] = __builtin_amdgcn_mfma_f32_16x16x4f32(aq[dj][s], bv, acc[t][dj], 0, 0, 0);
+                }
+            // sums over dj: output column 2 j + dj - 1 of pixel j; this lane's pixels are 2n (tile 0) and
+            // 2n+1 (tile 1), pixel 2n-1 is tile 1 of the lane to the left, pixel 2n+2 tile 0 of the lane to the right
+            float* rr = my_ring + (i % CT_RING) * CT_ROWF;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+            {
+                float4 v;
+                v.x = acc[0][1][r] + ct_from_left(acc[1][3][r]);                       // column 4n
+                v.y = acc[0][2][r] + ct_from_left(acc[1][4][r]) + acc[1][0][r];        // column 4n+1
+                v.z = acc[1][1][r] + acc[0][3][r];                                     // column 4n+2
+                v.w = acc[1][2][r] + acc[0][4][r] + ct_from_right(acc[0][0][r]);       // column 4n+3
+                *reinterpret_cast<float4*>(rr + (4 * kq + r) * 64 + 4 * l16) = v;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            if (i == row_a)
+            {
+#pragma unroll
+                for (int c = 0; c < 3; ++c) xfirst[wave][c * 64 + lane] = rr[c * 64 + lane];
+            }
+            if (i == row_b - 1)
+            {
+#pragma unroll
+                for (int c = 0; c < 6; ++c) xlast[wave][c * 64 + lane] = rr[(9 + c) * 64 + lane];
+            }
+            if (i > row_a)
+            {
+                // row i-1 is complete but for what a neighbouring wavefront holds
+                const float* rm = my_ring + ((i - 1) % CT_RING) * CT_ROWF;
+                float o[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                add_mid(rm, o);
+                if (i - 1 > row_a)
+                {
+                    const float* ru = my_ring + ((i - 2) % CT_RING) * CT_ROWF;
+                    add_up(ru + 9 * 64, ru + 12 * 64, o);
+                    add_down(rr, o);
+                    store(i - 1, o);
+                }
+                else
+                {
+                    add_down(rr, o);
+#pragma unroll
+                    for (int e = 0; e < 6; ++e) edge_first[e] = o[e];
+                }
+            }
+            if (i == row_b - 1)
+            {
+                float o[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                add_mid(rr, o);
+                if (i > row_a)
+                {
+                    const float* ru = my_ring + ((i - 1) % CT_RING) * CT_ROWF;
+                    add_up(ru + 9 * 64, ru + 12 * 64, o);
+                }
+#pragma unroll
+                for (int e = 0; e < 6; ++e) edge_last[e] = o[e];
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    b_cur[t][g] = b_next[t][g];
+        }
+        __syncthreads();
+        if (row_a < row_b)
+        {
+            // the wavefronts holding rows row_a - 1 and row_b (rows are dealt out in order, some wavefronts
+            // of a short strip get none)
+            int above = -1, below = -1;
+            for (int v = 0; v < CT_WAVES; ++v)
+            {
+                const int va = c0 + v * (c1 - c0) / CT_WAVES, vb = c0 + (v + 1) * (c1 - c0) / CT_WAVES;
+                if (va < vb && vb == row_a) above = v;
+                if (va < vb && va == row_b) below = v;
+            }
+            if (row_b - 1 > row_a)
+            {
+                if (above >= 0)
+                    add_up(&xlast[above][0], &xlast[above][3 * 64], edge_first);
+                store(row_a, edge_first);
+            }
+            else if (above >= 0)
+                add_up(&xlast[above][0], &xlast[above][3 * 64], edge_last);
+            if (below >= 0)
+                add_down(&xfirst[below][0], edge_last);
+            store(row_b - 1, edge_last);
+        }
+        __syncthreads();   // the next strip overwrites what the neighbours published
+    }
+}
+
 }  // namespace
 
 namespace dh
@@ -719,6 +981,39 @@ int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W,
 }
 
 
+
+
+// Returns 1 when the shape is not one dx_col2im takes (see the kernel's header), 0 after a launch.
+int conv_dx_col2im(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw, int C, int sh,
+                   int sw, int pt, int pl, int H, int W, const float* bias, int act, float alpha, hipStream_t st)
+{
+    const double dy_bytes = (double)N * Ho * Wo * O * 4.0;
+    if (sh != 2 || sw != 2 || kh != 5 || kw != 5 || pt != 1 || pl != 1 || C > 3 || O != 64 || Wo > CT_PIX || W != 2 * Wo ||
+        H != 2 * Ho || W > 64 || dy_bytes >= 4294967040.0 || (reinterpret_cast<uintptr_t>(dy) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(k) & 15) != 0)
+        return 1;
+    Col2imParams p{};
+    p.dy = dy; p.k = k; p.dx = dx; p.bias = bias; p.act = act; p.alpha = alpha;
+    p.N = N; p.Ho = Ho; p.Wo = Wo; p.C = C; p.H = H; p.W = W;
+    p.dy_bytes = (uint32_t)dy_bytes;
+    // rows per strip: whole images when those give every compute unit a workgroup, else the largest
+    // power of two that does (a strip computes two rows more than it owns)
+    int rows = 32;
+    while (rows > 4 && (long)N * ((Ho + rows - 1) / rows) < 1L * num_cus())
+        rows /= 2;
+    p.rows_per_strip = rows;
+    p.strips_per_image = (Ho + rows - 1) / rows;
+    const long strips = (long)N * p.strips_per_image;
+    if (strips > 0x7fffffffL)
+        return 1;
+    p.strips = (int)strips;
+    const long wgs = strips < num_cus() ? strips : num_cus();
+    const int prof = prof_begin("dx_col2im", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
+    hipLaunchKernelGGL(dx_col2im, dim3((unsigned)wgs), dim3(64 * CT_WAVES), 0, st, p);
+    prof_end(prof, st);
+    DH_LAUNCH_CHECK("dx_col2im launch");
+    return 0;
+}
 
 // Returns 1 when the shape is not one this kernel takes (the caller then uses the implicit GEMM),
 // 0 after a launch, or an error code.

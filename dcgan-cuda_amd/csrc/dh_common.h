@@ -54,6 +54,11 @@ struct ProfScope
 int conv_dx_few_channels(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw,
                          int C, int sh, int sw, int pt, int pl, int H, int W, const float* bias, int act,
                          float alpha, hipStream_t st);
+// The same product for the DCGAN's image layer (5x5, stride 2, at most 3 result channels, 64 dy channels,
+// dy rows of at most 32 pixels) as one dense product on the matrix cores followed by a scatter in LDS;
+// same return convention.  Tried before conv_dx_few_channels.
+int conv_dx_col2im(const float* dy, const float* k, float* dx, int N, int Ho, int Wo, int O, int kh, int kw, int C, int sh,
+                   int sw, int pt, int pl, int H, int W, const float* bias, int act, float alpha, hipStream_t st);
 // Forward convolution with a contraction of at most 80 (few input channels) and at most 64 output
 // channels, MFMA operands loaded straight from global memory; same return convention.
 int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
