@@ -47,19 +47,35 @@ CALIBRATION_COPY_BYTES = 256 << 20
 # summaries are kept under profiles/.  None = not measured.
 TRAFFIC_SOURCE = "profiles/bench_iteration_bs64_hbm_traffic.md"
 MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
-    # launch-weighted over the single and the paired instantiation of a tag
-    "conv_igemm_fast<dx,128x64>": 88.8e6,       # 9 single launches of 73.6 MB, 2 paired of 157.1 MB per iteration
-    "conv_igemm_fast<fwd,128x64>": 135.1e6,     # 6 x 119.9 MB, 1 x 226.3 MB
-    "conv_igemm_fast<dk,128x128>": 191.2e6,     # 3 x 126.1 MB, 3 x 256.2 MB
-    "conv_igemm_fast<fwd,128x128>": 182.0e6,    # 2 paired
-    "conv_igemm_fast<dx,128x128>": 171.3e6,     # 1 paired
-    "fwd_thin": 21.8e6,
-    "dk_thin": 35.8e6,     # launch-weighted: one paired launch (both towers) and one single per iteration
-    "dx_few_channels": 27.2e6,
+    # launch-weighted over the layer shapes and the single / paired instantiations of a tag
+    "conv_igemm_fast<dx,128x64>": 86.1e6,       # 9 single launches per iteration (35.6 / 93.2 / 88.6 MB), 2 paired (207.4 / 88.7 MB)
+    "conv_igemm_fast<fwd,128x64>": 146.4e6,     # 6 single (98.2 / 172.3 / 86.3 MB), 1 paired (309.8 MB)
+    "conv_igemm_fast<dk,128x128>": 191.4e6,     # 3 single (201.6 / 50.1 / 126.6 MB), 3 paired (402.1 / 261.2 / 106.7 MB)
+    "conv_igemm_fast<fwd,128x128>": 182.2e6,    # 2 paired
+    "conv_igemm_fast<dx,128x128>": 172.7e6,     # 1 paired
+    "fwd_thin": 21.7e6,
+    "dk_thin": 35.5e6,     # one paired launch (both towers) and one single per iteration
+    "dx_col2im": 23.5e6,
 }
 
 # DCGAN layers: (H, W, C, O) of the equivalent forward convolution, 5x5, stride 2, SAME
 LAYERS = [(64, 64, 3, 64), (32, 32, 64, 128), (16, 16, 128, 256), (8, 8, 256, 512)]
+
+
+def hbm_row(r, steps):
+    """One memory-bound kernel class of the second pass.  A class whose launches move under 1 MiB (the
+    64-element bias gradient of the dense head: 256 bytes) is launch latency and nothing else: it is
+    listed with its time and without a bandwidth figure."""
+    per_launch = r["flops"] / r["launches"]
+    row = {"name": r["name"][4:], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+           "bytes_per_launch": round(per_launch), "ms_per_step": round(r["ms"] / steps, 4)}
+    if per_launch >= (1 << 20):
+        row["gbs"] = round(r["flops"] / (r["ms"] * 1e-3) / 1e9, 3)
+        row["frac"] = round(r["flops"] / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)
+    else:
+        row["gbs"] = row["frac"] = None
+        row["note"] = "launch-latency bound: %d bytes per launch" % round(per_launch)
+    return row
 
 
 def conv_flops(batch, layer):
@@ -545,11 +561,7 @@ def main():
                      "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2),
                      "frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
                      "issued_frac": issued_frac(r)} for r in sorted(rows, key=lambda r: -r["ms"])],
-        "hbm_kernels": [{"name": r["name"][4:], "launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
-                         "bytes_per_launch": round(r["flops"] / r["launches"]),
-                         "gbs": round(r["flops"] / (r["ms"] * 1e-3) / 1e9, 3),
-                         "frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
-                         "ms_per_step": round(r["ms"] / aux_steps, 4)} for r in sorted(hbm_rows, key=lambda r: -r["ms"])],
+        "hbm_kernels": [hbm_row(r, aux_steps) for r in sorted(hbm_rows, key=lambda r: -r["ms"])],
         "dense_gemm": [{"launches": r["launches"], "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
                         "ms_per_step": round(r["ms"] / aux_steps, 4)} for r in dense_rows],
         "hbm_kernels_note": "measured in %d extra iterations after the timed region, algorithmic bytes / "

@@ -970,7 +970,8 @@ int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W,
     const long resident = 2L * num_cus();
     if (blocks > resident)
         blocks = resident;
-    const int prof = prof_begin("fwd_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
+    const int prof = prof_begin("fwd_thin", 2.0 * N * Ho * Wo * O * kh * kw * C, st, 1,
+                                (double)tiles * TF_KH * TF_NB * 4096.0);   // 32x32x2 MFMAs issued, padding included
     if (kw * C <= 16 && kh * 16 <= 2 * TF_KH)
         hipLaunchKernelGGL(fwd_thin<true>, dim3((unsigned)blocks), dim3(256), 0, st, p);
     else
@@ -1008,7 +1009,11 @@ int conv_dx_col2im(const float* dy, const float* k, float* dx, int N, int Ho, in
         return 1;
     p.strips = (int)strips;
     const long wgs = strips < num_cus() ? strips : num_cus();
-    const int prof = prof_begin("dx_col2im", 2.0 * N * Ho * Wo * O * kh * kw * C, st);
+    // rows of Z computed, the strips' extra rows included: 160 MFMAs of 16x16x4 each
+    long z_rows = 0;
+    for (int r0 = 0; r0 < Ho; r0 += rows)
+        z_rows += (r0 + rows + 1 < Ho ? r0 + rows + 1 : Ho) - (r0 > 0 ? r0 - 1 : 0);
+    const int prof = prof_begin("dx_col2im", 2.0 * N * Ho * Wo * O * kh * kw * C, st, 1, (double)N * z_rows * 160.0 * 2048.0);
     hipLaunchKernelGGL(dx_col2im, dim3((unsigned)wgs), dim3(64 * CT_WAVES), 0, st, p);
     prof_end(prof, st);
     DH_LAUNCH_CHECK("dx_col2im launch");
@@ -1118,7 +1123,8 @@ int conv_dk_thin(const float* x, const float* dy, const float* x2, const float* 
     void* ws;
     DH_TRY(workspace((size_t)wgs * M * O * sizeof(float), &ws, st));
     p.part = static_cast<float*>(ws);
-    const int prof = prof_begin("dk_thin", 2.0 * images * Ho * Wo * O * kh * kw * C, st);
+    const int prof = prof_begin("dk_thin", 2.0 * images * Ho * Wo * O * kh * kw * C, st, 1,
+                                2.0 * images * Ho * Wo * (DT_MT * 16.0) * (DT_NT * 16.0));   // the 80 x 64 tile per pixel
     hipLaunchKernelGGL(dk_thin, dim3((unsigned)wgs), dim3(64 * DT_WAVES), 0, st, p);
     prof_end(prof, st);
     DH_LAUNCH_CHECK("dk_thin launch");
