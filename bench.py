@@ -54,6 +54,7 @@ MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FET
     "conv_igemm_fast<fwd,128x128>": 182.2e6,    # 2 paired
     "conv_igemm_fast<dx,128x128>": 172.7e6,     # 1 paired
     "fwd_thin": 21.7e6,
+    "fwd_rows": 21.7e6,    # same tensors as fwd_thin, which it replaces on the DCGAN shape
     "dk_thin": 35.5e6,     # one paired launch (both towers) and one single per iteration
     "dx_col2im": 23.5e6,
 }

@@ -675,6 +675,225 @@ __global__ __launch_bounds__(64 * DT_WAVES, 2) void dk_thin(const ThinDkParams p
     }
 }
 
+// ---- forward from three channels, a row of output pixels per step ---------------------------------
+// The same product as fwd_thin, [N,64,64,3] -> [N,32,32,64] with a 5x5 filter, organised so that next
+// to the MFMAs almost no vector instruction is left (fp32 MFMAs and vector instructions share the
+// SIMD's ALU: fwd_thin issues ~470 of them per 32 pixels for offsets, masks and selects).
+//   * y^T = K^T * patches: the filter is the A operand (80 registers per lane for the whole kernel:
+//     four tiles of 16 output channels x the contraction 5 filter rows x 16), the patches are B, so
+//     that result lane (pixel, q) holds 4 consecutive channels of its pixel: 16-byte stores.
+//   * The contraction index is (di, e) with e = dj*C + c = 0 .. 14: the 15 values of a filter row's
+//     taps are 15 CONSECUTIVE floats of input row i*sh + di - pad, starting at ((j*sw - pad)*C).  A
+//     wavefront parks the input rows of its task (4 output rows: 11 input rows, 8.4 KB that are
+//     contiguous in memory and are loaded as such, 16 bytes per lane) in LDS of its own, every row
+//     with zeros to its left and right and rows outside the image as zeros, and each lane reads its
+//     operand values from there with an address that is a per-lane constant plus the row's base:
+//     20 LDS reads per 16 pixels, no masks, no bounds checks.
+//   * The sixteenth slot of filter row 0 carries the bias (operand value 1), of the other rows zero.
+//   * No wavefront depends on another: no barrier.  Tasks are strided over persistent wavefronts, the
+//     loads of the next task are issued before the MFMAs of this one and waited for after the first
+//     row's MFMAs, before any store of this task is issued (the counter of outstanding memory
+//     operations is in order and counts stores).
+// Takes kh = 5, kw*C = 15, at most 64 output channels in multiples of 16, rows of at most 32 output
+// pixels; other shapes keep fwd_thin.
+// Reference counterpart: kernel_conv2d (src/gpu/conv2d.cu:13-62) with kernel_mat_rvect_add and the
+// activation that follow it.
+typedef unsigned int fr_u32x4 __attribute__((__vector_size__(16)));
+constexpr int FR_WAVES = 8;
+constexpr int FR_STAGED = 11;           // input rows of a task: (4 - 1) * 2 + 5
+constexpr int FR_RS = 208;              // floats per parked row: 8 of zeros, up to 192 of data, zeros
+constexpr int FR_LEFT = 8;
+constexpr int FR_LOADS = 9;
+constexpr int FR_ACT_LEAKY01 = 5;       // leaky relu with a slope in [0, 1]: max(v, slope * v), the same value in two instructions             // 16-byte loads per lane and task: 11 rows x 48 <= 9 x 64
+
+struct FwdRowsParams
+{
+    const float* x;
+    const float* k;
+    const float* bias;
+    float* y;
+    float alpha;
+    int N, H, W, C, Ho, Wo, O, sh, sw, pt, pl;
+    int rows_per_task, tasks_per_image, tasks;
+    int staged, chunks_per_row;         // input rows of a task; 16-byte chunks of an input row
+    uint32_t x_bytes, y_bytes;
+};
+
+template <int ACT>
+__global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams p)
+{
+    __shared__ __attribute__((aligned(16))) float parked[FR_WAVES][(FR_STAGED + 1) * FR_RS];   // (+1: where surplus lanes write)
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l16 = lane & 15, kq = lane >> 4;
+    float* const my = &parked[wave][0];
+    for (int e = 4 * lane; e < (FR_STAGED + 1) * FR_RS; e += 256)
+        *reinterpret_cast<float4*>(my + e) = make_float4(0.f, 0.f, 0.f, 0.f);
+
+    // A[m = channel 16 mt + l16][k = 16 di + 4 u + kq] of MFMA step 4 di + u (loads without a branch:
+    // what does not exist is out of the descriptor's range and reads as zero)
+    constexpr uint32_t FAR = 0xffffff00u;
+    float aq[4][20];
+    {
+        const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.k), 0, 75 * p.O * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.bias), 0, p.bias ? p.O * 4 : 0, 0x00020000);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+        {
+            const int o = 16 * mt + l16;
+#pragma unroll
+            for (int s = 0; s < 20; ++s)
+            {
+                const int di = s >> 2, e = 4 * (s & 3) + kq;
+                const bool ok = (int)(o < p.O) & (int)(e < 15);
+                aq[mt][s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(kr, (int)(ok ? (uint32_t)((di * 15 + e) * p.O + o) * 4u : FAR), 0, 0));
+            }
+            const float bv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, (int)(o < p.O ? (uint32_t)o * 4u : FAR), 0, 0));
+            aq[mt][3] = kq == 3 ? bv : aq[mt][3];
+        }
+    }
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)p.y_bytes, 0x00020000);
+    // chunk t*64 + lane of a task's rows: its row and where it is parked
+    int put[FR_LOADS], chunk_row[FR_LOADS];
+#pragma unroll
+    for (int t = 0; t < FR_LOADS; ++t)
+    {
+        const int q = t * 64 + lane;
+        const int r = q / p.chunks_per_row;
+        chunk_row[t] = r < p.staged ? r : -0x10000;         // surplus chunks: loaded as zeros ...
+        put[t] = r < p.staged ? r * FR_RS + FR_LEFT + 4 * (q - r * p.chunks_per_row)
+                              : FR_STAGED * FR_RS + 4 * (lane & 31);                 // ... and parked out of the way
+    }
+    // this lane's operand values of pixel 16 t + l16: floats 4u + kq from here in the parked row
+    int take[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+        take[t] = FR_LEFT + ((16 * t + l16) * p.sw - p.pl) * p.C + kq;
+    const float slot15_row0 = p.bias ? 1.f : 0.f;
+    const uint32_t row_bytes = (uint32_t)p.W * p.C * 4u;
+
+    auto issue = [&](int task, dt_f32x4 (&raw)[FR_LOADS]) {
+        const int b = task / p.tasks_per_image;
+        const int h0 = (task - b * p.tasks_per_image) * p.rows_per_task * p.sh - p.pt;
+        const uint32_t base = ((uint32_t)b * p.H + (uint32_t)h0) * row_bytes;        // (wraps for h0 < 0; such rows are not loaded)
+#pragma unroll
+        for (int t = 0; t < FR_LOADS; ++t)
+        {
+            const int h = h0 + chunk_row[t];
+            const bool ok = (int)(task < p.tasks) & (int)(h >= 0) & (int)(h < p.H);
+            raw[t] = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(ok ? base + (uint32_t)(t * 64 + lane) * 16u : FAR), 0, 0));
+        }
+    };
+    auto park = [&](const dt_f32x4 (&raw)[FR_LOADS]) {
+#pragma unroll
+        for (int t = 0; t < FR_LOADS; ++t)
+            *reinterpret_cast<dt_f32x4*>(my + put[t]) = raw[t];
+    };
+
+    const int stride = gridDim.x * FR_WAVES;
+    int task = blockIdx.x * FR_WAVES + wave;
+    dt_f32x4 raw[FR_LOADS];
+    issue(task, raw);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    park(raw);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (; task < p.tasks; task += stride)
+    {
+        issue(task + stride, raw);
+        __builtin_amdgcn_sched_barrier(0);      // (the scheduler would sink the loads to where they are used)
+        const int b = task / p.tasks_per_image;
+        const int i0 = (task - b * p.tasks_per_image) * p.rows_per_task;
+#pragma unroll
+        for (int ii = 0; ii < 4; ++ii)
+        {
+            if (ii < p.rows_per_task && i0 + ii < p.Ho)
+            {
+                dt_f32x4 acc[2][4];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            acc[t][mt][r] = 0.f;
+                // operand values of filter row di: 4 floats per pixel tile, read one filter row ahead of
+                // the MFMAs that consume them (left to itself the scheduler puts every read right in front
+                // of its first use and the wavefront waits out the LDS latency twenty times per row)
+                auto fetch = [&](int di, float (&v)[2][4]) {
+                    const float* row = my + (ii * p.sh + di) * FR_RS;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                    {
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+                            v[t][u] = row[take[t] + 4 * u];
+                    }
+                };
+                float bv[5][2][4];
+                fetch(0, bv[0]);
+#pragma unroll
+                for (int di = 0; di < 5; ++di)
+                {
+                    if (di + 1 < 5)
+                        fetch(di + 1, bv[di + 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                    {
+                        if (kq == 3)
+                            bv[di][t][3] = di == 0 ? slot15_row0 : 0.f;
+#pragma unroll
+                        for (int u = 0; u < 4; ++u)
+#pragma unroll
+                            for (int mt = 0; mt < 4; ++mt)
+                                acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(aq[mt][4 * di + u], bv[di][t][u], acc[t][mt], 0, 0, 0);
+                    }
+                }
+                if (ii == 0)
+                {
+                    // the next task's rows have had these MFMAs to arrive; no store of this task is out yet
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int t = 0; t < FR_LOADS; ++t)
+                        asm volatile("" : "+v"(raw[t]));
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // lane (pixel, q) holds channels 16 mt + 4 q .. + 3 of its pixel
+                const uint32_t row_off = (((uint32_t)b * p.Ho + (uint32_t)(i0 + ii)) * p.Wo) * (uint32_t)p.O * 4u;
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                {
+                    const int j = 16 * t + l16;
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt)
+                    {
+                        dt_f32x4 v = acc[t][mt];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                        {
+                            if (ACT == DH_ACT_RELU) v[r] = v[r] < 0.f ? 0.f : v[r];
+                            else if (ACT == DH_ACT_LEAKY) v[r] = v[r] < 0.f ? p.alpha * v[r] : v[r];
+                            else if (ACT == FR_ACT_LEAKY01) v[r] = fmaxf(v[r], p.alpha * v[r]);
+                            else if (ACT == DH_ACT_TANH) v[r] = tanhf(v[r]);
+                            else if (ACT == DH_ACT_SIGMOID) v[r] = 1.f / (1.f + expf(-v[r]));
+                        }
+                        const bool ok = (int)(j < p.Wo) & (int)(16 * mt + 4 * kq < p.O);
+                        const uint32_t off = row_off + ((uint32_t)j * p.O + 16u * mt + 4u * kq) * 4u;
+                        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(fr_u32x4, v), yr, (int)(ok ? off : FAR), 0, 0);
+                    }
+                }
+            }
+        }
+        // the rows of this task have been read: the next task's take their place
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        park(raw);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 // ---- transposed convolution onto few channels as a product followed by in-register sums ----------
 // The generator's image layer, [N,32,32,64] -> [N,64,64,3] (5x5, stride 2), and the gradient of the
 // discriminator's first layer.  Written as dx[b, 2i+di-1, 2j+dj-1, c] += Z[(b,i,j), (di,dj,c)] with
@@ -942,11 +1161,66 @@ __global__ __launch_bounds__(64 * CT_WAVES, 2) void dx_col2im(const Col2imParams
 namespace dh
 {
 
+// Returns 1 when the shape is not one fwd_rows takes (see the kernel's header), 0 after a launch.
+int conv_fwd_rows(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
+                  int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st)
+{
+    const double x_bytes = (double)N * H * W * C * 4.0, y_bytes = (double)N * Ho * Wo * O * 4.0;
+    if (kh != 5 || kw * C != 15 || O > 64 || O % 16 != 0 || Wo > 32 || sh < 1 || sh > 2 || sw < 1 || sw > 2 || pt < 0 ||
+        pl < 0 || pl * C > FR_LEFT || (W * C) % 4 != 0 || W * C > FR_RS - FR_LEFT - 8 ||
+        FR_LEFT + (31 * sw - pl) * C + 16 > FR_RS || act < DH_ACT_NONE || act > DH_ACT_SIGMOID ||
+        x_bytes >= 4294967040.0 || y_bytes >= 4294967040.0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(y) & 15) != 0)
+        return 1;
+    FwdRowsParams p{};
+    p.x = x; p.k = k; p.bias = bias; p.y = y; p.alpha = alpha;
+    p.N = N; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.O = O; p.sh = sh; p.sw = sw; p.pt = pt; p.pl = pl;
+    p.x_bytes = (uint32_t)x_bytes; p.y_bytes = (uint32_t)y_bytes;
+    p.chunks_per_row = W * C / 4;
+    // output rows per task: four (they share input rows) when that still gives every wavefront slot a task
+    const long slots = (long)num_cus() * FR_WAVES;
+    int rows = 4;
+    while (rows > 1 && (long)N * ((Ho + rows - 1) / rows) < slots)
+        rows /= 2;
+    p.rows_per_task = rows;
+    p.staged = (rows - 1) * sh + 5;
+    if (p.staged > FR_STAGED || p.staged * p.chunks_per_row > FR_LOADS * 64)
+        return 1;
+    p.tasks_per_image = (Ho + rows - 1) / rows;
+    const long tasks = (long)N * p.tasks_per_image;
+    if (tasks > 0x3fffffffL)
+        return 1;
+    p.tasks = (int)tasks;
+    long wgs = (tasks + FR_WAVES - 1) / FR_WAVES;
+    if (wgs > num_cus())
+        wgs = num_cus();
+    const int prof = prof_begin("fwd_rows", 2.0 * N * Ho * Wo * O * kh * kw * C, st, 1, (double)N * Ho * 160.0 * 2048.0);
+    const dim3 grid((unsigned)wgs), block(64 * FR_WAVES);
+    switch (act)
+    {
+    case DH_ACT_NONE: hipLaunchKernelGGL(fwd_rows<DH_ACT_NONE>, grid, block, 0, st, p); break;
+    case DH_ACT_RELU: hipLaunchKernelGGL(fwd_rows<DH_ACT_RELU>, grid, block, 0, st, p); break;
+    case DH_ACT_LEAKY:
+        if (alpha >= 0.f && alpha <= 1.f)
+            hipLaunchKernelGGL(fwd_rows<FR_ACT_LEAKY01>, grid, block, 0, st, p);
+        else
+            hipLaunchKernelGGL(fwd_rows<DH_ACT_LEAKY>, grid, block, 0, st, p);
+        break;
+    case DH_ACT_TANH: hipLaunchKernelGGL(fwd_rows<DH_ACT_TANH>, grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL(fwd_rows<DH_ACT_SIGMOID>, grid, block, 0, st, p); break;
+    }
+    prof_end(prof, st);
+    DH_LAUNCH_CHECK("fwd_rows launch");
+    return 0;
+}
+
 // Returns 1 when the shape is not one this kernel takes (the caller then uses the implicit GEMM),
 // 0 after a launch, or an error code.
 int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
                   int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st)
 {
+    if (conv_fwd_rows(x, k, y, N, H, W, C, kh, kw, O, sh, sw, pt, pl, Ho, Wo, bias, act, alpha, st) == 0)
+        return 0;
     const long K = (long)kh * kw * C;
     const size_t x_bytes = (size_t)N * H * W * C * 4;
     if (K > 2 * TF_KH || C > 4 || O > 32 * TF_NB || O % 4 != 0 || x_bytes >= (size_t(1) << 31) ||

@@ -164,6 +164,44 @@ def test_fwd_from_few_channels(be, orc, shape):
         be.lib.dh_debug_force_generic_conv(0)
 
 
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (2, 64, 64, 3, 5, 5, 64, 2),       # one output row per task
+    (130, 64, 64, 3, 5, 5, 16, 2),     # two output rows per task
+    (264, 60, 64, 3, 5, 5, 64, 2),     # four, the last task of an image two; 30 output rows
+    (64, 128, 32, 3, 5, 5, 32, 1),     # stride 1 (two pixels of padding), four rows per task
+    (3, 20, 12, 3, 5, 5, 48, 2),       # rows of 6 output pixels, 48 channels
+    (2, 64, 64, 1, 5, 15, 16, 2),      # one channel, a filter row of 15 taps
+])
+def test_fwd_from_three_channels_row_by_row(be, orc, shape):
+    """The row-wise forward kernel (5 filter rows of 15 values; bias carried in the 16th slot of the
+    contraction, input rows parked in LDS with zeros around them) against the oracle, with the fused
+    bias + activation epilogues and without, at every number of output rows per task."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(37, *shape)
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    orc.set_threads(8)
+    plain = orc.conv2d(x, k, (s, s))
+    close(be.conv2d(x, k, (s, s)), plain, what="no epilogue")
+    biased = orc.bias_add(plain, bias)
+    close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2), orc.relu_leaky(biased, 0.2), what="bias + leaky")
+    close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=1.5), orc.relu_leaky(biased, 1.5), what="bias + leaky, slope > 1")
+    if N <= 3:
+        close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_TANH), orc.tanh(biased), what="bias + tanh")
+        close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_RELU), orc.relu(biased), what="bias + relu")
+        close(be.conv2d(x, k, (s, s), bias=bias, act=A.ACT_SIGMOID), orc.sigmoid(biased), what="bias + sigmoid")
+    A.profile_enable(1)
+    A.profile_reset()
+    try:
+        be.conv2d(x, k, (s, s))
+        tags = [r["name"] for r in A.profile_read()]
+    finally:
+        A.profile_enable(0)
+    assert tags == ["fwd_rows"], tags
+
+
 @pytest.mark.parametrize("shape", [(2, 64, 64, 3, 5, 5, 64, 2), (1, 9, 11, 3, 5, 5, 8, 2), (2, 12, 14, 4, 4, 5, 24, 1)])
 def test_fwd_from_few_channels_reads_only_its_taps(be, orc, shape):
     """The thin forward kernel loads 16 bytes at a time and discards the elements that belong to no tap
