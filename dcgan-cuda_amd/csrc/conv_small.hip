@@ -723,6 +723,7 @@ template <int ACT>
 __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams p)
 {
     __shared__ __attribute__((aligned(16))) float parked[FR_WAVES][(FR_STAGED + 1) * FR_RS];   // (+1: where surplus lanes write)
+    __shared__ __attribute__((aligned(16))) float filt[77 * 64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l16 = lane & 15, kq = lane >> 4;
@@ -730,28 +731,35 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
     for (int e = 4 * lane; e < (FR_STAGED + 1) * FR_RS; e += 256)
         *reinterpret_cast<float4*>(my + e) = make_float4(0.f, 0.f, 0.f, 0.f);
 
-    // A[m = channel 16 mt + l16][k = 16 di + 4 u + kq] of MFMA step 4 di + u (loads without a branch:
-    // what does not exist is out of the descriptor's range and reads as zero)
+    // The filter goes through LDS once per workgroup: 16-byte loads of the [75][O] matrix as it lies in
+    // memory (row 75: the bias, row 76 and the columns from O on: zeros -- what does not exist is out of
+    // the descriptors' range and reads as zero), then every lane picks its 80 values (fetched by each
+    // lane itself they would be 84 four-byte loads per lane of every wavefront).
     constexpr uint32_t FAR = 0xffffff00u;
-    float aq[4][20];
     {
         const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.k), 0, 75 * p.O * 4, 0x00020000);
         const __amdgpu_buffer_rsrc_t br = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.bias), 0, p.bias ? p.O * 4 : 0, 0x00020000);
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int slot = threadIdx.x; slot < 77 * 16; slot += 64 * FR_WAVES)
         {
-            const int o = 16 * mt + l16;
-#pragma unroll
-            for (int s = 0; s < 20; ++s)
-            {
-                const int di = s >> 2, e = 4 * (s & 3) + kq;
-                const bool ok = (int)(o < p.O) & (int)(e < 15);
-                aq[mt][s] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(kr, (int)(ok ? (uint32_t)((di * 15 + e) * p.O + o) * 4u : FAR), 0, 0));
-            }
-            const float bv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, (int)(o < p.O ? (uint32_t)o * 4u : FAR), 0, 0));
-            aq[mt][3] = kq == 3 ? bv : aq[mt][3];
+            const int row = slot >> 4, col = 4 * (slot & 15);
+            const bool in_k = (int)(row < 75) & (int)(col < p.O), in_b = (int)(row == 75) & (int)(col < p.O);
+            const dt_f32x4 kv = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(kr, (int)(in_k ? (uint32_t)(row * p.O + col) * 4u : FAR), 0, 0));
+            const dt_f32x4 bv = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(br, (int)(in_b ? (uint32_t)col * 4u : FAR), 0, 0));
+            *reinterpret_cast<dt_f32x4*>(&filt[row * 64 + col]) = row == 75 ? bv : kv;
         }
     }
+    __syncthreads();
+    // A[m = channel 16 mt + l16][k = 16 di + 4 u + kq] of MFMA step 4 di + u
+    float aq[4][20];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int s = 0; s < 20; ++s)
+        {
+            const int di = s >> 2, e = 4 * (s & 3) + kq;
+            const int row = e < 15 ? di * 15 + e : (di == 0 ? 75 : 76);
+            aq[mt][s] = filt[row * 64 + 16 * mt + l16];
+        }
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)p.y_bytes, 0x00020000);
     // chunk t*64 + lane of a task's rows: its row and where it is parked
