@@ -977,27 +977,29 @@ __global__ __launch_bounds__(64 * CT_WAVES, 2) void dx_col2im(const Col2imParams
     const int l16 = lane & 15, kq = lane >> 4;
 
     // the filter as MFMA operand A[m = (di,c)][k = o] of tile dj: lane (m, q) holds o = 16q .. 16q+15
+    // (rows that do not exist are out of the descriptor's range and read as zero: no select, and no wait
+    // for the filter before the first row's loads go out)
+    constexpr uint32_t FAR = 0xffffff00u;
     float aq[5][CT_KS];
     {
+        const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.k), 0, 25 * p.C * 64 * 4, 0x00020000);
         const int di = l16 / 3, c = l16 - 3 * di;
-        const bool ok = l16 < 15 && c < p.C;
+        const bool ok = (int)(l16 < 15) & (int)(c < p.C);
 #pragma unroll
         for (int dj = 0; dj < 5; ++dj)
         {
-            const float* src = p.k + (size_t)(ok ? (di * 5 + dj) * p.C + c : 0) * 64 + kq * 16;
+            const uint32_t off = (uint32_t)(((di * 5 + dj) * p.C + c) * 64 + kq * 16) * 4u;
 #pragma unroll
             for (int g = 0; g < 4; ++g)
             {
-                const float4 v = *reinterpret_cast<const float4*>(src + 4 * g);
-                aq[dj][4 * g + 0] = ok ? v.x : 0.f; aq[dj][4 * g + 1] = ok ? v.y : 0.f;
-                aq[dj][4 * g + 2] = ok ? v.z : 0.f; aq[dj][4 * g + 3] = ok ? v.w : 0.f;
+                const dt_f32x4 v = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(kr, (int)(ok ? off + 16u * g : FAR), 0, 0));
+                aq[dj][4 * g + 0] = v[0]; aq[dj][4 * g + 1] = v[1]; aq[dj][4 * g + 2] = v[2]; aq[dj][4 * g + 3] = v[3];
             }
         }
     }
     const float bias_c[3] = {p.bias && p.C > 0 ? p.bias[0] : 0.f, p.bias && p.C > 1 ? p.bias[1] : 0.f,
                              p.bias && p.C > 2 ? p.bias[2] : 0.f};
     const __amdgpu_buffer_rsrc_t dr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.dy), 0, (int)p.dy_bytes, 0x00020000);
-    constexpr uint32_t FAR = 0xffffff00u;
     float* const my_ring = &ring[wave][0][0];
 
     for (int strip = blockIdx.x; strip < p.strips; strip += gridDim.x)

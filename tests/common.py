@@ -13,9 +13,12 @@ RTOL, ATOL = 1e-4, 1e-5
 def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
     """The two-sided parity check of the batch-64 suites.  `exp32` is the oracle's fp32 result (the
     reference's arithmetic and summation order), `exp64` the same computed with float64 sums.
-      * element by element: |got - exp32| <= 1e-4 |exp32| + 1e-5 max(1, max|exp32|) -- the stated fp32
-        tolerance, its absolute part widened for tensors of large magnitude (sums of thousands of O(1)
-        products cannot be held to 1e-5 by any fp32 summation order);
+      * element by element: |got - exp32| <= 1e-4 |exp32| + max(1e-5 max(1, max|exp32|), 3 max|exp32 - exp64|)
+        -- the stated fp32 tolerance, its absolute part widened for tensors of large magnitude (sums of
+        thousands of O(1) products cannot be held to 1e-5 by any fp32 summation order) and never below
+        three times the oracle's OWN distance from the float64 result: the reference's serial fp32 sum
+        over 65 536 rows (the first layer's bias gradient) is itself 1.4e-5 away from the exact sum, and
+        a result that is 3e-8 from exact must not fail for disagreeing with it;
       * against the float64 result, with the oracle's own fp32 rounding error as the yardstick:
         max |got - exp64| <= max(2 * slack * max |exp32 - exp64|, 1e-5 * min(1, max|exp32|)) -- the
         floor follows the magnitude downwards, so that gradients of magnitude 1e-6 are not waved
@@ -37,7 +40,7 @@ def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
     print("%-50s max|exp| %.3g  oracle32-f64 %.3g  gpu-f64 %.3g  ratio %.2f" % (what, mag, yard, err, err / max(yard, 1e-30)),
           flush=True)
     if elementwise:
-        np.testing.assert_allclose(got, exp32, rtol=RTOL, atol=ATOL * max(1.0, mag), err_msg=what)
+        np.testing.assert_allclose(got, exp32, rtol=RTOL, atol=max(ATOL * max(1.0, mag), 3.0 * yard), err_msg=what)
     if kinks and exp32.size:
         l2 = float(np.linalg.norm(got - exp64) / max(np.linalg.norm(exp64), 1e-30))
         assert l2 <= 1e-3, "%s: relative L2 error %.3g" % (what, l2)
