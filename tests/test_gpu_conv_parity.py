@@ -133,6 +133,39 @@ def test_dx_onto_few_channels(be, orc, shape):
 
 
 @pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
+    (130, 64, 64, 3, 5, 5, 64, 2),     # strips of 16 rows: a row above and below each computed twice
+    (264, 64, 64, 2, 5, 5, 64, 2),     # whole images, two channels
+    (70, 20, 24, 1, 5, 5, 64, 2),      # strips of 4 of 10 rows, rows of 12 pixels, one channel
+    (300, 20, 24, 3, 5, 5, 64, 2),     # whole images of 10 rows on eight wavefronts
+    (40, 44, 64, 3, 5, 5, 64, 2),      # 22 rows in strips of 4: a last strip of 2
+])
+def test_dx_onto_three_channels_by_rows(be, orc, shape):
+    """The matrix-core transposed convolution onto 1-3 channels (one dense product per dy row, sums over
+    filter columns in registers, down the rows through LDS; wavefronts exchanging edge rows) at every
+    strip height, with the fused bias + tanh and without, repeatable to the bit."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(47, *shape)
+    bias_c = np.linspace(-0.3, 0.3, C).astype(np.float32)
+    orc.set_threads(8)
+    plain = orc.conv2d_input_grad(dy, k, s, (H, W))
+    A.profile_enable(1)
+    A.profile_reset()
+    try:
+        got = be.conv2d_input_grad(dy, k, s, (H, W))
+        tags = [r["name"] for r in A.profile_read()]
+    finally:
+        A.profile_enable(0)
+    assert tags == ["dx_col2im"], tags
+    close(got, plain, what="no epilogue")
+    np.testing.assert_array_equal(got, be.conv2d_input_grad(dy, k, s, (H, W)))
+    close(be.conv2d_input_grad(dy, k, s, (H, W), bias=bias_c, act=A.ACT_TANH), orc.tanh(orc.bias_add(plain, bias_c)),
+          what="bias + tanh")
+
+
+@pytest.mark.parametrize("shape", [  # N, H, W, C, kh, kw, O, stride
     (2, 64, 64, 3, 5, 5, 64, 2),     # the discriminator's first layer, batch 2
     (3, 19, 13, 1, 5, 5, 16, 2),     # ragged tiles on both axes, one channel
     (2, 70, 37, 2, 3, 3, 48, 2),     # more than one tile along both axes, three blocks of output channels
