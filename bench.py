@@ -41,23 +41,34 @@ PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_GBS = 8000.0
 CALIBRATION_COPY_BYTES = 256 << 20
 
-# HBM bytes per launch of the convolution kernels in the batch-64 iteration, from two
-# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE; averages over the launches of
-# one kernel symbol), each scaled by the same counter's reading for the calibration copy.  The
-# summaries are kept under profiles/.  None = not measured.
+# HBM bytes per launch of the convolution kernels in the batch-64 iteration come from two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE), each scaled by the same counter's
+# reading for the calibration copy.  The summary of those runs is kept under profiles/ and is READ here
+# (not pasted): regenerating the profile updates the figure, a missing file gives `traffic: null`.
 TRAFFIC_SOURCE = "profiles/bench_iteration_bs64_hbm_traffic.md"
-MEASURED_TRAFFIC_BYTES = {   # profiles/bench_iteration_bs64_hbm_traffic.md (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000),
-    # launch-weighted over the layer shapes and the single / paired instantiations of a tag
-    "conv_igemm_fast<dx,128x64>": 86.1e6,       # 9 single launches per iteration (35.6 / 93.2 / 88.6 MB), 2 paired (207.4 / 88.7 MB)
-    "conv_igemm_fast<fwd,128x64>": 146.4e6,     # 6 single (98.2 / 172.3 / 86.3 MB), 1 paired (309.8 MB)
-    "conv_igemm_fast<dk,128x128>": 191.4e6,     # 3 single (201.6 / 50.1 / 126.6 MB), 3 paired (402.1 / 261.2 / 106.7 MB)
-    "conv_igemm_fast<fwd,128x128>": 182.2e6,    # 2 paired
-    "conv_igemm_fast<dx,128x128>": 172.7e6,     # 1 paired
-    "fwd_thin": 21.7e6,
-    "fwd_rows": 21.7e6,    # same tensors as fwd_thin, which it replaces on the DCGAN shape
-    "dk_thin": 35.5e6,     # one paired launch (both towers) and one single per iteration
-    "dx_col2im": 23.5e6,
-}
+
+
+def measured_traffic_bytes():
+    """{kernel tag: HBM bytes per launch}, launch-weighted over the layer shapes and the single / paired
+    instantiations that share a tag, from the table of TRAFFIC_SOURCE (columns: kernel, workgroups,
+    launches, FETCH_SIZE KiB, WRITE_SIZE KiB, scaled read MB, scaled write MB, total MB, GB/s)."""
+    import re
+    path = os.path.join(ROOT, TRAFFIC_SOURCE)
+    if not os.path.exists(path):
+        return {}
+    total, launches = {}, {}
+    for line in open(path):
+        if not line.startswith("| `"):
+            continue
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        name, n, mb = cells[0].strip("`"), int(cells[2]), float(cells[7])
+        m = re.match(r"conv_igemm_fast<(\d), (\d+), (\d+), \d, \d, \w+>", name)
+        tag = ("conv_igemm_fast<%s,%sx%s>" % (("fwd", "dx", "dk")[int(m.group(1))], m.group(2), m.group(3))) if m \
+            else name.split("<")[0]
+        total[tag] = total.get(tag, 0.0) + n * mb * 1e6
+        launches[tag] = launches.get(tag, 0) + n
+    return {tag: total[tag] / launches[tag] for tag in total}
+
 
 # DCGAN layers: (H, W, C, O) of the equivalent forward convolution, 5x5, stride 2, SAME
 LAYERS = [(64, 64, 3, 64), (32, 32, 64, 128), (16, 16, 128, 256), (8, 8, 256, 512)]
@@ -539,7 +550,8 @@ def main():
     conv_fl = sum(r["flops"] for r in rows)
     dom = max(rows, key=lambda r: r["ms"])
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
-    traffic = MEASURED_TRAFFIC_BYTES.get(dom["name"]) if args.batch == 64 else None
+    traffic = measured_traffic_bytes().get(dom["name"]) if args.batch == 64 else None
+    traffic = round(traffic) if traffic else None
 
     def issued_frac(r):
         """Matrix-core utilisation proper: the FLOPs the kernel issues (live k-slabs as full tiles --
