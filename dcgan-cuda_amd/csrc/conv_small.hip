@@ -703,8 +703,9 @@ constexpr int FR_WAVES = 8;
 constexpr int FR_STAGED = 11;           // input rows of a task: (4 - 1) * 2 + 5
 constexpr int FR_RS = 208;              // floats per parked row: 8 of zeros, up to 192 of data, zeros
 constexpr int FR_LEFT = 8;
-constexpr int FR_LOADS = 9;
-constexpr int FR_ACT_LEAKY01 = 5;       // leaky relu with a slope in [0, 1]: max(v, slope * v), the same value in two instructions             // 16-byte loads per lane and task: 11 rows x 48 <= 9 x 64
+constexpr int FR_LOADS = 9;             // 16-byte loads per lane and task: 11 rows x 48 <= 9 x 64
+constexpr int FR_HEAD = 4;              // the first of them hold input rows 0 .. 4: 5 x 48 <= 4 x 64
+constexpr int FR_ACT_LEAKY01 = 5;       // leaky relu with a slope in [0, 1]: max(v, slope * v), the same value in two instructions
 
 struct FwdRowsParams
 {
@@ -793,23 +794,30 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
             raw[t] = __builtin_bit_cast(dt_f32x4, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(ok ? base + (uint32_t)(t * 64 + lane) * 16u : FAR), 0, 0));
         }
     };
-    auto park = [&](const dt_f32x4 (&raw)[FR_LOADS]) {
+    auto park = [&](const dt_f32x4 (&raw)[FR_LOADS], int from, int to) {
 #pragma unroll
         for (int t = 0; t < FR_LOADS; ++t)
-            *reinterpret_cast<dt_f32x4*>(my + put[t]) = raw[t];
+            if (t >= from && t < to)
+                *reinterpret_cast<dt_f32x4*>(my + put[t]) = raw[t];
     };
 
     const int stride = gridDim.x * FR_WAVES;
     int task = blockIdx.x * FR_WAVES + wave;
     dt_f32x4 raw[FR_LOADS];
+    // The first task: every wavefront of the device asks for its rows at the same moment, and until they
+    // arrive there is nothing to multiply.  Output row 0 needs input rows 0 .. 4 only, which the first
+    // FR_HEAD loads hold (5 rows of at most 48 chunks); they are parked as soon as THEY are there, and the
+    // rest of the task's rows after the first row's MFMAs.
     issue(task, raw);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    park(raw);
+    park(raw, 0, FR_HEAD);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    bool first_task = true;
     for (; task < p.tasks; task += stride)
     {
-        issue(task + stride, raw);
+        if (!first_task)
+            issue(task + stride, raw);
         __builtin_amdgcn_sched_barrier(0);      // (the scheduler would sink the loads to where they are used)
         const int b = task / p.tasks_per_image;
         const int i0 = (task - b * p.tasks_per_image) * p.rows_per_task;
@@ -861,11 +869,24 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
                 }
                 if (ii == 0)
                 {
-                    // the next task's rows have had these MFMAs to arrive; no store of this task is out yet
                     __builtin_amdgcn_sched_barrier(0);
+                    if (first_task)
+                    {
+                        // the rest of this task's rows, then the request for the next task's
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        park(raw, FR_HEAD, FR_LOADS);
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        issue(task + stride, raw);
+                        first_task = false;
+                    }
+                    else
+                    {
+                        // the next task's rows have had these MFMAs to arrive; no store of this task is out yet
 #pragma unroll
-                    for (int t = 0; t < FR_LOADS; ++t)
-                        asm volatile("" : "+v"(raw[t]));
+                        for (int t = 0; t < FR_LOADS; ++t)
+                            asm volatile("" : "+v"(raw[t]));
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // lane (pixel, q) holds channels 16 mt + 4 q .. + 3 of its pixel
@@ -896,7 +917,7 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
         }
         // the rows of this task have been read: the next task's take their place
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        park(raw);
+        park(raw, 0, FR_LOADS);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
