@@ -102,21 +102,27 @@ void ORC(conv2d)(const float* x, const float* k, float* y,
         const int j = (int)(r % Wo);
         const int i = (int)((r / Wo) % Ho);
         const int b = (int)(r / ((long)Wo * Ho));
+        /* The sums of the O output channels do not touch each other: they advance side by side
+         * (o innermost, where filter and output are contiguous), each in the reference's order. */
+        acc_t val[O > 0 ? O : 1];
         for (int o = 0; o < O; ++o)
-        {
-            acc_t val = 0;
-            for (int c = 0; c < C; ++c)
-                for (int di = 0; di < kh; ++di)
-                    for (int dj = 0; dj < kw; ++dj)
+            val[o] = 0;
+        for (int c = 0; c < C; ++c)
+            for (int di = 0; di < kh; ++di)
+                for (int dj = 0; dj < kw; ++dj)
+                {
+                    const int h = sh * i + di - pt;
+                    const int w = sw * j + dj - pl;
+                    if (h >= 0 && w >= 0 && h < H && w < W)
                     {
-                        const int h = sh * i + di - pt;
-                        const int w = sw * j + dj - pl;
-                        if (h >= 0 && w >= 0 && h < H && w < W)
-                            val += x[(((size_t)b * H + h) * W + w) * C + c]
-                                 * k[(((size_t)di * kw + dj) * C + c) * O + o];
+                        const float xv = x[(((size_t)b * H + h) * W + w) * C + c];
+                        const float* kr = k + (((size_t)di * kw + dj) * C + c) * O;
+                        for (int o = 0; o < O; ++o)
+                            val[o] += xv * kr[o];
                     }
-            y[(size_t)r * O + o] = (float)val;
-        }
+                }
+        for (int o = 0; o < O; ++o)
+            y[(size_t)r * O + o] = (float)val[o];
     }
 }
 
@@ -150,26 +156,31 @@ void ORC(conv2d_input_grad)(const float* dy, const float* k, float* dx,
         const int b = (int)(r / ((long)W * H));
         for (int c = 0; c < C; ++c)
         {
+            /* one sum per filter, advanced side by side (f innermost: dy and k are contiguous in
+             * f), each over (kernel row, kernel column) in the reference's order; then the sums are
+             * added in filter order */
+            acc_t val[O > 0 ? O : 1];
+            for (int f = 0; f < O; ++f)
+                val[f] = 0;
+            for (int a = 0; a < kh; ++a)
+            {
+                const int th = h + a - pad_top;
+                if (th < 0 || th % stride != 0 || th / stride >= Ho)
+                    continue;
+                for (int e = 0; e < kw; ++e)
+                {
+                    const int tw = w + e - pad_left;
+                    if (tw < 0 || tw % stride != 0 || tw / stride >= Wo)
+                        continue;
+                    const float* dr = dy + (((size_t)b * Ho + th / stride) * Wo + tw / stride) * O;
+                    const float* kr = k + (((size_t)(kh - 1 - a) * kw + (kw - 1 - e)) * C + c) * O;
+                    for (int f = 0; f < O; ++f)
+                        val[f] += dr[f] * kr[f];
+                }
+            }
             acc_t total = 0;
             for (int f = 0; f < O; ++f)
-            {
-                acc_t val = 0;
-                for (int a = 0; a < kh; ++a)
-                {
-                    const int th = h + a - pad_top;
-                    if (th < 0 || th % stride != 0 || th / stride >= Ho)
-                        continue;
-                    for (int e = 0; e < kw; ++e)
-                    {
-                        const int tw = w + e - pad_left;
-                        if (tw < 0 || tw % stride != 0 || tw / stride >= Wo)
-                            continue;
-                        val += dy[(((size_t)b * Ho + th / stride) * Wo + tw / stride) * O + f]
-                             * k[(((size_t)(kh - 1 - a) * kw + (kw - 1 - e)) * C + c) * O + f];
-                    }
-                }
-                total = (f == 0) ? val : total + val;
-            }
+                total = (f == 0) ? val[f] : total + val[f];
             dx[(size_t)r * C + c] = (float)total;
         }
     }
@@ -201,30 +212,37 @@ void ORC(conv2d_kernel_grad)(const float* dy, const float* x, float* dk,
         const int c = (int)(r % C);
         const int dj = (int)((r / C) % kw);
         const int di = (int)(r / ((long)C * kw));
+        /* one sum per output channel, advanced side by side (o innermost: dy and dk are contiguous
+         * in o), each over (output row, output column) of one image in the reference's order; the
+         * per-image sums are added in image order */
+        acc_t total[O > 0 ? O : 1], val[O > 0 ? O : 1];
         for (int o = 0; o < O; ++o)
+            total[o] = 0;
+        for (int b = 0; b < N; ++b)
         {
-            acc_t total = 0;
-            for (int b = 0; b < N; ++b)
+            for (int o = 0; o < O; ++o)
+                val[o] = 0;
+            for (int i = 0; i < Ho; ++i)
             {
-                acc_t val = 0;
-                for (int i = 0; i < Ho; ++i)
+                const int h = di + stride * i - pt;
+                if (h < 0 || h >= H)
+                    continue;
+                for (int j = 0; j < Wo; ++j)
                 {
-                    const int h = di + stride * i - pt;
-                    if (h < 0 || h >= H)
+                    const int w = dj + stride * j - pl;
+                    if (w < 0 || w >= W)
                         continue;
-                    for (int j = 0; j < Wo; ++j)
-                    {
-                        const int w = dj + stride * j - pl;
-                        if (w < 0 || w >= W)
-                            continue;
-                        val += x[(((size_t)b * H + h) * W + w) * C + c]
-                             * dy[(((size_t)b * Ho + i) * Wo + j) * O + o];
-                    }
+                    const float xv = x[(((size_t)b * H + h) * W + w) * C + c];
+                    const float* dr = dy + (((size_t)b * Ho + i) * Wo + j) * O;
+                    for (int o = 0; o < O; ++o)
+                        val[o] += xv * dr[o];
                 }
-                total = (b == 0) ? val : total + val;
             }
-            dk[(size_t)r * O + o] = (float)total;
+            for (int o = 0; o < O; ++o)
+                total[o] = (b == 0) ? val[o] : total[o] + val[o];
         }
+        for (int o = 0; o < O; ++o)
+            dk[(size_t)r * O + o] = (float)total[o];
     }
 }
 
