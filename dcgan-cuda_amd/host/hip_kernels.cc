@@ -24,7 +24,7 @@ namespace
 {
 
 int g_fusion = -1;         // -1: not decided yet (reads DCGAN_HIP_FUSE)
-int g_last_launches = 0;    // steps of the plan that ran last
+int g_last_launches = 0;    // steps of the plan that ran last and launched something
 bool g_pairing = true;     // issue same-filter convolutions of independent towers as one launch (part of fusion)
 
 #define CK(call) hip_check((call), #call)
@@ -63,6 +63,7 @@ struct Step
     // inside the optimiser launch (defer_bias_sums).  Producer (ACT_BIAS_GRAD, or NODE mat_sum_cols):
     // where the sums go.  ADAM: for each of its two gradient slots, the sums and their count.
     dbl_t* parts = nullptr;
+    bool rows_as_parts = false;   // NODE mat_sum_cols of a matrix of few rows: no launch, the optimiser adds the rows up
     const dbl_t* g_parts[2] = {nullptr, nullptr};
     std::size_t g_nparts[2] = {0, 0};
 };
@@ -196,6 +197,24 @@ dbl_t* parts_buffer(const dbl_t* grad, std::size_t floats)
     return slot.first;
 }
 
+// Whether exactly one node of the plan writes the tensor.
+bool written_once(const Plan& plan, const dbl_t* t)
+{
+    int writers = 0;
+    auto count = [&](const Step& s) {
+        for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+            if (n && (n->out1 == t || n->out2 == t))
+                writers += 1;
+    };
+    for (const Step& s : plan.steps)
+    {
+        count(s);
+        for (const Step& g : s.group)
+            count(g);
+    }
+    return writers == 1;
+}
+
 void defer_bias_sums(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
 {
     // the optimiser steps of the plan, by address
@@ -249,13 +268,25 @@ void defer_bias_sums(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
                     ok = false;
         if (!ok)
             continue;
-        const std::size_t nparts = dh_bias_grad_part_count(sum->len1, sum->len2);
-        if (nparts < 2)
+        std::size_t nparts = dh_bias_grad_part_count(sum->len1, sum->len2);
+        const dbl_t* sums = nullptr;
+        if (nparts >= 2)
+            sums = s.parts = parts_buffer(db, nparts * sum->len2);
+        else if (s.kind == Step::NODE && sum->len1 >= 2 && sum->len1 <= 256 && written_once(plan, sum->in1))
+        {
+            // A matrix of few rows (the dense head's [batch x 1] logit gradients) is its own list of
+            // row-range sums, one row each: the column-sum launches (two one-workgroup kernels, ~4.6 us
+            // each whatever they do) go away and the optimiser launch adds the rows up.  The matrix is
+            // written by one step only, so it still holds these values when the optimiser runs.
+            s.rows_as_parts = true;
+            sums = sum->in1;
+            nparts = sum->len1;
+        }
+        else
             continue;
-        s.parts = parts_buffer(db, nparts * sum->len2);
         for (auto& sl : slots)
         {
-            sl.first->g_parts[sl.second] = s.parts;
+            sl.first->g_parts[sl.second] = sums;
             sl.first->g_nparts[sl.second] = nparts;
         }
     }
@@ -753,6 +784,8 @@ void issue(const Step& s)
                 CK(dh_leaky_relu_grad(s.act_ref, n->in2, n->out1, n->cons1, n->len1, g_stream));
             return;
         }
+        if (s.rows_as_parts)
+            return;   // the optimiser launch reads the rows themselves
         if (s.parts)
         {
             // bias gradient left as row-range sums for the optimiser launch
@@ -992,7 +1025,9 @@ void run_async(rt::NodesList& tasks)
     }
     // inputs the run did not touch: the caller's buffers are only borrowed until the run returns
     flush_feeds(nullptr);
-    g_last_launches = (int)it->second.steps.size();
+    g_last_launches = 0;
+    for (const Step& s : it->second.steps)
+        g_last_launches += s.rows_as_parts ? 0 : 1;
 }
 
 int last_launch_count() { return g_last_launches; }
