@@ -159,6 +159,9 @@ __global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, 
                     acc[r] = fmaf(x[u][r], w[u], acc[r]);
         };
         int k = 0;
+        if (RPT <= 4)   // registers allow sixteen k in flight: a contraction of 64 or 100 is 4 or 7 round trips, not 16 or 25
+            for (; k + 16 <= K; k += 16)
+                block(k, std::integral_constant<int, 16>{});
         for (; k + 4 <= K; k += 4)
             block(k, std::integral_constant<int, 4>{});
         for (; k < K; ++k)
@@ -172,6 +175,44 @@ __global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, 
                 out[(size_t)i * out_si + (size_t)j * out_sj] = acc[r] + bj;
         }
     }
+}
+
+// out[j] = sum_k a[k*sak] * B[k*sbk + j] (+ bias[j]): a vector times a matrix with contiguous rows (the
+// filter gradient of the 8192 -> 1 layer: 64 logit gradients times the [64 x 8192] activations).  A
+// workgroup owns 64 columns; its four wavefronts take a quarter of the contraction each, sixteen loads in
+// flight per lane, and wavefront 0 adds the four partial sums in a fixed order.  (gemm_skinny<1> walks
+// the whole contraction in one wavefront, four loads at a time, while three wavefronts idle: 10 us
+// against 5 for this shape.)
+__global__ __launch_bounds__(256) void gemv_rows(const float* __restrict__ a, const float* __restrict__ b,
+                                                 const float* __restrict__ bias, float* __restrict__ out, int K, int P,
+                                                 size_t sak, size_t sbk)
+{
+    __shared__ float part[4][64];
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const int j = blockIdx.x * 64 + tx;
+    const int jc = j < P ? j : P - 1;
+    const int kq = (K + 3) / 4;
+    const int k0 = ty * kq, k1 = K < k0 + kq ? K : k0 + kq;
+    float s = 0.f;
+    for (int k = k0; k < k1; k += 16)
+    {
+        float w[16], x[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+        {
+            const bool live = k + u < k1;
+            const int kk = live ? k + u : k0;   // a valid row; its product is dropped
+            w[u] = b[(size_t)kk * sbk + jc];
+            x[u] = live ? a[(size_t)kk * sak] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            s = fmaf(x[u], w[u], s);
+    }
+    part[ty][tx] = s;
+    __syncthreads();
+    if (ty == 0 && j < P)
+        out[j] = ((part[0][tx] + part[1][tx]) + part[2][tx]) + part[3][tx] + (bias ? bias[j] : 0.f);
 }
 
 // one workgroup per output element: 256 lanes stride over k, then a fixed LDS tree
@@ -228,14 +269,15 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     else if (n <= SK_MAXK && sbj == 1 && p >= 64 && m > 4)
         hipLaunchKernelGGL(gemm_skinny<16>, dim3((unsigned)((p + 63) / 64), (unsigned)((m + 63) / 64)), dim3(256), 0, st, a, b,
                            bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+    else if (n <= SK_MAXK && sbj == 1 && p >= 64 && m == 1)
+        hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((p + 63) / 64)), dim3(256), 0, st, a, b, bias, out, (int)n, (int)p, sak, sbk);
     else if (n <= SK_MAXK && sbj == 1 && p >= 64)
         hipLaunchKernelGGL(gemm_skinny<1>, dim3((unsigned)((p + 63) / 64), 1u), dim3(256), 0, st, a, b, bias, out, (int)m,
                            (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
     else if (n <= SK_MAXK && p == 1 && sai == 1 && !bias && m >= 64)
         // a single output column: out[i] = sum_k a[k*sak + i] * b[k*sbk] is the row vector b times the
         // matrix a, whose rows are contiguous -- the same kernel with the roles exchanged
-        hipLaunchKernelGGL(gemm_skinny<1>, dim3((unsigned)((m + 63) / 64), 1u), dim3(256), 0, st, b, a, bias, out, 1, (int)n,
-                           (int)m, (size_t)0, sbk, sak, (size_t)0, (size_t)1);
+        hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((m + 63) / 64)), dim3(256), 0, st, b, a, bias, out, (int)n, (int)m, sbk, sak);
     else if (m * p <= 16384 && n >= 512)
         hipLaunchKernelGGL(gemm_block_per_output, dim3((unsigned)(m * p)), dim3(256), 0, st, a, b, bias, out,
                            (int)m, (int)n, (int)p, sai, sak, sbk, sbj);

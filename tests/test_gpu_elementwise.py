@@ -95,8 +95,11 @@ def test_argmax_is_exact(be, orc):
         assert be.argmax_acc(y, yh) == orc.argmax_acc(y, yh)
 
 
+# (1, n, p) and (m, n, 1): a vector times a matrix, contraction cut over four wavefronts (whole sixteens, a ragged
+# last quarter, fewer rows than wavefronts)
 @pytest.mark.parametrize("m,n,p", [(64, 100, 8192), (64, 8192, 1), (9, 33, 17), (1, 1, 1), (130, 70, 65), (64, 128, 200), (3, 5, 64),
-                                   (200, 129, 70)])
+                                   (200, 129, 70), (1, 64, 8192), (1, 37, 100), (1, 128, 65), (1, 3, 64), (37, 200, 1),
+                                   (128, 64, 1)])
 def test_dense(be, orc, m, n, p):
     rng = np.random.default_rng(m + n + p)
     x = rng.uniform(-1, 1, (m, n)).astype(np.float32)
