@@ -62,7 +62,7 @@ def measured_traffic_bytes():
             continue
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
         name, n, mb = cells[0].strip("`"), int(cells[2]), float(cells[7])
-        m = re.match(r"conv_igemm_fast<(\d), (\d+), (\d+), \d, \d, \w+>", name)
+        m = re.match(r"conv_igemm_fast<(\d), (\d+), (\d+), \d, \d(?:, \w+)+>", name)
         tag = ("conv_igemm_fast<%s,%sx%s>" % (("fwd", "dx", "dk")[int(m.group(1))], m.group(2), m.group(3))) if m \
             else name.split("<")[0]
         total[tag] = total.get(tag, 0.0) + n * mb * 1e6
@@ -551,6 +551,8 @@ def main():
     dom = max(rows, key=lambda r: r["ms"])
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
     traffic = measured_traffic_bytes().get(dom["name"]) if args.batch == 64 else None
+    if args.batch == 64 and traffic is None:
+        print("bench.py: %s has no row for %s; roofline.traffic is null" % (TRAFFIC_SOURCE, dom["name"]), file=sys.stderr)
     traffic = round(traffic) if traffic else None
 
     def issued_frac(r):
