@@ -114,13 +114,32 @@ def test_dcgan_layers_losses_gradients_and_one_adam_iteration(cpu_dump, fusion):
             np.testing.assert_allclose(g, exp, rtol=RTOL, atol=ATOL * scale, err_msg=key)
 
 
-def agree_with_yardstick(key, got, exp32, exp64):
+def kinks_between(got, exp32):
+    """Layer outputs (relu / leaky-relu) that are positive in one run and not in the other although both are at
+    the rounding level: the pre-activation sum came out on either side of zero, and every gradient that
+    passes through that element takes a different slope in the two runs."""
+    found = 0
+    for key in got:
+        if key.startswith(("d_fake_l", "d_real_l")) or (key.startswith("g_l") and key != "g_l4"):
+            g, e = np.asarray(got[key]).reshape(-1), np.asarray(exp32[key]).reshape(-1)
+            if g.size != e.size:       # a tiled batch: its first copy
+                g = g[:e.size]
+            flipped = ((g > 0) != (e > 0)) & (np.abs(g) < 1e-6) & (np.abs(e) < 1e-6)
+            if flipped.any():
+                print("%-50s %d output(s) on the other side of zero at the rounding level" % (key, int(flipped.sum())), flush=True)
+            found += int(flipped.sum())
+    return found
+
+
+def agree_with_yardstick(key, got, exp32, exp64, kinks=0):
     """common.agree with slack 3 (every tensor of the network lies downstream of an input-gradient
-    product).  Parameters after Adam steps additionally: a step is ~ lr * sign(gradient) while the second
+    product); gradients get the allowance for activation kinks only when kinks_between found one.
+    Parameters after Adam steps additionally: a step is ~ lr * sign(gradient) while the second
     moment is young, so a gradient at the rounding level flips the step of single elements in either
     fp32 run (the yardstick then is a whole step); such elements must be as rare as in the oracle's own
     fp32 run."""
-    agree(got, exp32, exp64, key, slack=3.0, elementwise=not key.startswith("after_"), kinks=key.startswith("grad_"))
+    agree(got, exp32, exp64, key, slack=3.0, elementwise=not key.startswith("after_"),
+          kinks=kinks > 0 and key.startswith("grad_"))
     if key.startswith("after_"):
         got, exp32, exp64 = (np.asarray(a, np.float64).reshape(-1) for a in (got, exp32, exp64))
         frac = float(np.mean(np.abs(got - exp64) > 1e-6))      # a step is 2e-4
@@ -138,8 +157,9 @@ def test_training_iterations_at_batch_64(cpu_dump64, cpu_dump64_f64, fusion):
     print("fusion", fusion, flush=True)
     got, _ = gpu_dump(fusion, batch=64, steps=3, one_run=True)
     assert set(got) == set(cpu_dump64)
+    kinks = kinks_between(got, cpu_dump64)
     for key in sorted(cpu_dump64):
-        agree_with_yardstick(key, got[key], cpu_dump64[key], cpu_dump64_f64[key])
+        agree_with_yardstick(key, got[key], cpu_dump64[key], cpu_dump64_f64[key], kinks)
 
 
 def test_fused_plans_at_batch_64_tensor_by_tensor(cpu_dump64, cpu_dump64_f64):
@@ -155,9 +175,11 @@ def test_fused_plans_at_batch_64_tensor_by_tensor(cpu_dump64, cpu_dump64_f64):
             model.set_var(name, val)
         model.set_inputs(z, x)
         names = dict(dr.tensor_names())
+        layers = [br + "_l%d" % i for br in ("d_fake", "d_real") for i in range(4)] + ["g_l%d" % i for i in range(4)]
+        kinks = kinks_between({key: model.eval(names[key]) for key in layers}, cpu_dump64)
         for key in ("g_out", "d_fake_l3", "d_real_logits", "d_loss", "g_loss", "grad_d_loss_d0_w", "grad_d_loss_d3_w",
                     "grad_d_loss_d2_b", "grad_g_loss_g1_w", "grad_g_loss_g4_w", "grad_g_loss_g0_b", "grad_g_loss_x_fake"):
-            agree_with_yardstick(key, model.eval(names[key]), cpu_dump64[key], cpu_dump64_f64[key])
+            agree_with_yardstick(key, model.eval(names[key]), cpu_dump64[key], cpu_dump64_f64[key], kinks)
     finally:
         model.set_fusion(False)
         model.close()
@@ -172,6 +194,7 @@ def test_iteration_at_batch_512_repeats_the_batch_64_one(cpu_dump64, cpu_dump64_
                  "grad_g_loss_x_fake": 12288}
     for br in ("d_fake", "d_real"):
         per_image.update({br + "_l0": 65536, br + "_l1": 32768, br + "_l2": 16384, br + "_l3": 8192, br + "_logits": 1})
+    kinks = kinks_between(got, cpu_dump64)
     for key in sorted(cpu_dump64):
         g = got[key]
         if key in per_image:
@@ -181,9 +204,9 @@ def test_iteration_at_batch_512_repeats_the_batch_64_one(cpu_dump64, cpu_dump64_
                                            err_msg="%s, copy %d" % (key, rep))
             g = g[0]
             if key == "grad_g_loss_x_fake":   # gradient of a mean over 8 times the images
-                agree_with_yardstick(key, g, cpu_dump64[key] / 8.0, cpu_dump64_f64[key] / 8.0)
+                agree_with_yardstick(key, g, cpu_dump64[key] / 8.0, cpu_dump64_f64[key] / 8.0, kinks)
                 continue
-        agree_with_yardstick(key, g, cpu_dump64[key], cpu_dump64_f64[key])
+        agree_with_yardstick(key, g, cpu_dump64[key], cpu_dump64_f64[key], kinks)
 
 
 def test_generate_and_argmax_bit_exact(cpu_dump):
