@@ -540,6 +540,29 @@ def main():
         model.g_step(z=z)          # graph.run({g_opti, g_loss}, {z}) and the loss read back
     ref_wall = time.perf_counter() - t1
 
+    # What a drop-in behind the reference's seams gets, under the conditions of `value` (inputs resident, no
+    # loss read back): node by node through the kernel table (the shim that replaces src/gpu/kernels.cu and
+    # runner.cu, nothing else), and the planner when Graph::run hands it the instruction list and nothing
+    # else -- gpu::run's own signature -- so that it has to keep every intermediate tensor.  `value` is the
+    # planner with the tensors read back named by Graph::run (one added call in src/ops/graph.cu).
+    def rate(setup):
+        setup()
+        for _ in range(3):
+            iteration()
+        model.sync()
+        t = time.perf_counter()
+        for _ in range(ref_steps):
+            iteration()
+        model.sync()
+        return ref_steps / (time.perf_counter() - t)
+
+    table_rate = rate(lambda: model.set_fusion(False))
+    table_launches = model.last_launch_count()
+    list_only_rate = rate(lambda: (model.set_fusion(True), model.set_name_results(False)))
+    list_only_launches = model.last_launch_count()
+    model.set_name_results(True)
+    model.set_fusion(bool(args.fusion))
+
     calibration_copy(A)
 
     ms_per_step = wall * 1e3 / args.steps
@@ -600,6 +623,18 @@ def main():
                            "ms_per_step": round(ref_wall * 1e3 / ref_steps, 4),
                            "what": "the reference's own training loop (dcgan/main.cu:378-397): z and the image batch fed "
                                    "from pageable host memory and both losses read back in every iteration"},
+        "table_runner_value": round(table_rate, 3),
+        "drop_in": {
+            "unit": "iterations/s", "steps": ref_steps,
+            "table_runner": {"value": round(table_rate, 3), "launches_in_g_step": table_launches,
+                             "what": "every instruction through hip::kernels_list[node->type], in list order, one "
+                                     "wait per run: the shim for src/gpu/kernels.cu + runner.cu and no other change"},
+            "planner_list_only": {"value": round(list_only_rate, 3), "launches_in_g_step": list_only_launches,
+                                  "what": "hip::run(NodesList&) as src/ops/graph.cu:199 calls gpu::run, nothing said "
+                                          "about the tensors read afterwards: only fusions that keep every tensor"},
+            "planner_results_named": {"value": round(args.steps / wall, 3),
+                                      "what": "`value`: Graph::run names the tensors it reads back "
+                                              "(hip::set_protected_tensors) before the run"}},
         "device": A.device_info(),
         "roofline": roofline,
     }

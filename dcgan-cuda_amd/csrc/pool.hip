@@ -166,10 +166,13 @@ int dh_pool_reserve(size_t bytes)
     DH_TRY(current_device(&dev));
     std::lock_guard<std::mutex> lock(g_pool_mu);
     Pool& p = g_pool[dev];
-    const size_t idle = p.held - p.in_use;
-    if (bytes <= idle) return 0;
-    const size_t want = (bytes - idle + ALIGN - 1) / ALIGN * ALIGN;
-    return add_slab(p, want);
+    // one idle range of that size, not idle bytes in total: fragments do not serve a large request
+    const size_t need = bytes == 0 ? ALIGN : (bytes + ALIGN - 1) / ALIGN * ALIGN;
+    if (need < bytes) return fail(DH_EINVAL, "dh_pool_reserve: size overflows");
+    int slab = -1;
+    size_t offset = 0;
+    if (best_fit(p, need, &slab, &offset)) return 0;
+    return add_slab(p, need);
 }
 
 int dh_pool_trim(void)

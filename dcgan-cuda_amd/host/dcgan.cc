@@ -264,6 +264,12 @@ void dg_set_fusion(int fuse)
     hip::forget_plans();
 }
 
+void dg_set_name_results(int on)
+{
+    ops::Graph::instance().name_results_set(on != 0);
+    hip::forget_plans();
+}
+
 void dg_set_pairing(int on)
 {
     hip::set_pairing(on != 0);

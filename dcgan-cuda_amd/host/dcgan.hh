@@ -49,6 +49,10 @@ void dg_destroy(void* model);
 void dg_set_fusion(int fuse);
 // on != 0 (the default): with fusion, same-filter convolutions of independent towers run as one paired launch.
 void dg_set_pairing(int on);
+// on == 0: every run hands the backend its instruction list and nothing else, as the reference's Graph::run
+// does (src/ops/graph.cu:194-200), so the planner keeps every intermediate tensor; on != 0 (the default): the
+// run names the tensors it reads back and the others may be left out.
+void dg_set_name_results(int on);
 // Variables in the order g conv-transpose 1..4 (w,b), g dense (w,b), d conv 0..3 (w,b), d dense (w,b).
 int dg_num_vars(void* model);
 long dg_var_size(void* model, int index);

@@ -1,7 +1,10 @@
 // The HIP backend's planning runner: the instruction list of a run is pattern-matched into fused and
 // paired C-ABI calls (or issued node by node through the kernel table of hip_table.cc when fusion is
 // off), without the reference's per-node device synchronisation (src/gpu/runner.cu:10-18).
-#include "backend.hh"
+//
+// Depends on rt::Node, rt::NodesList and the C ABI only (see hip_runner.hh): it compiles unchanged
+// against the reference's src/runtime headers.
+#include "hip_runner.hh"
 
 #include <algorithm>
 #include <cmath>
@@ -15,7 +18,6 @@
 #include <unordered_set>
 
 #include "dcgan_hip.h"
-#include "memory.hh"
 
 namespace hip
 {
@@ -27,7 +29,7 @@ int g_fusion = -1;         // -1: not decided yet (reads DCGAN_HIP_FUSE)
 int g_last_launches = 0;    // steps of the plan that ran last and launched something
 bool g_pairing = true;     // issue same-filter convolutions of independent towers as one launch (part of fusion)
 
-#define CK(call) hip_check((call), #call)
+#define CK(call) check((call), #call)
 
 // conv_fwd / conv_dx: one C-ABI call for a decoded geometry (with optional epilogue)
 void conv_fwd(const ConvGeom& g, const dbl_t* x, const dbl_t* k, dbl_t* y, const dbl_t* bias, int act, float alpha)
@@ -89,6 +91,17 @@ bool is_conv_like(const rt::Node* n)
 struct Plan
 {
     std::vector<Step> steps;
+};
+
+// The tensors the caller may read once the run is over.  gpu::run receives nothing but the instruction
+// list (src/gpu/runner.cu:10, src/ops/graph.cu:194-215 reads the results afterwards), so until the
+// caller has named them with set_protected_tensors EVERY tensor counts: the plan then holds only the
+// fusions that still write all outputs of the nodes they stand for.
+struct Keep
+{
+    bool all = true;
+    std::unordered_set<const dbl_t*> set;
+    std::size_t count(const dbl_t* t) const { return all || set.count(t) ? 1 : 0; }
 };
 
 // Which instructions of the list read tensor `t`.
@@ -215,7 +228,7 @@ bool written_once(const Plan& plan, const dbl_t* t)
     return writers == 1;
 }
 
-void defer_bias_sums(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
+void defer_bias_sums(Plan& plan, const Keep& keep)
 {
     // the optimiser steps of the plan, by address
     std::vector<Step*> adams;
@@ -407,7 +420,7 @@ void inputs_of(const Step& s, std::vector<const dbl_t*>& in)
         inputs_of(g, in);
 }
 
-void pair_convolutions(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
+void pair_convolutions(Plan& plan, const Keep& keep)
 {
     std::vector<Step>& st = plan.steps;
     int n = 0;   // the steps before the first one that writes a variable in place may be re-ordered
@@ -553,7 +566,7 @@ void pair_convolutions(Plan& plan, const std::unordered_set<const dbl_t*>& keep)
     st.swap(order);
 }
 
-Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<const dbl_t*>& keep, bool fuse)
+Plan make_plan(const std::vector<rt::Node*>& nodes, const Keep& keep, bool fuse)
 {
     Plan plan;
     if (!fuse)
@@ -572,12 +585,13 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
     std::unordered_map<const dbl_t*, const dbl_t*> z_alias;
     std::unordered_map<rt::Node*, Step> fused_at;  // fused step keyed by the LAST node it replaces
 
-    auto only_reader = [&](const dbl_t* t, rt::Node* who) {
-        if (keep.count(t))
-            return false;
+    // the one instruction of the list that reads t
+    auto sole_reader = [&](const dbl_t* t, rt::Node* who) {
         const auto& r = readers.of(t);
         return r.size() == 1 && r[0] == who;
     };
+    // ... and the caller does not read it either: t need not exist after the run
+    auto only_reader = [&](const dbl_t* t, rt::Node* who) { return !keep.count(t) && sole_reader(t, who); };
 
     for (rt::Node* n : nodes)
     {
@@ -673,8 +687,9 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
                 if (p->type == rt::Node::OP_MOMENT_UPDATE2 && p->out1 == n->in2) m2 = p;
             }
             if (m1 && m2 && m1->in1 == m2->in1 && m1->len1 == n->len1 && m2->len1 == n->len1 &&
-                !absorbed.count(m1) && !absorbed.count(m2) && only_reader(m1->out1, n) && only_reader(m2->out1, n))
+                !absorbed.count(m1) && !absorbed.count(m2) && sole_reader(m1->out1, n) && sole_reader(m2->out1, n))
             {
+                // (the single pass writes both moments and the variable: nothing the caller could read is lost)
                 Step s;
                 s.kind = Step::ADAM;
                 s.node = n;
@@ -744,7 +759,7 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const std::unordered_set<con
         static const char* kinds[] = {"node", "conv+epilogue", "act-grad+bias-grad", "adam", "adam-multi", "conv pair"};
         std::fprintf(stderr, "plan of %zu nodes -> %zu steps\n", nodes.size(), plan.steps.size());
         for (const Step& s : plan.steps)
-            std::fprintf(stderr, "  %-20s %-32s len %zu\n", kinds[s.kind], rt::Node::name_of(s.node->type),
+            std::fprintf(stderr, "  %-20s %-32s len %zu\n", kinds[s.kind], op_name(s.node->type),
                          (std::size_t)s.node->len1);
     }
     return plan;
@@ -794,7 +809,7 @@ void issue(const Step& s)
         }
         kernel_f f = n->type >= 0 && n->type < 512 ? kernels_list[n->type] : nullptr;
         if (!f)
-            throw std::runtime_error(std::string("hip backend: operator '") + rt::Node::name_of(n->type) +
+            throw std::runtime_error(std::string("hip backend: operator '") + op_name(n->type) +
                                      "' is not on the convolution path and has no HIP kernel");
         f(n);
         return;
@@ -881,14 +896,18 @@ struct PlanKey
 {
     std::vector<rt::Node*> nodes;
     std::vector<const dbl_t*> keep;  // sorted
+    bool keep_all;
     bool fuse;
-    bool operator==(const PlanKey& o) const { return fuse == o.fuse && nodes == o.nodes && keep == o.keep; }
+    bool operator==(const PlanKey& o) const
+    {
+        return fuse == o.fuse && keep_all == o.keep_all && nodes == o.nodes && keep == o.keep;
+    }
 };
 struct PlanKeyHash
 {
     std::size_t operator()(const PlanKey& k) const
     {
-        std::size_t h = k.fuse ? 0x9e3779b97f4a7c15ull : 0;
+        std::size_t h = (k.fuse ? 0x9e3779b97f4a7c15ull : 0) + (k.keep_all ? 1 : 0);
         for (rt::Node* n : k.nodes)
             h = (h ^ reinterpret_cast<std::size_t>(n)) * 0x100000001b3ull;
         for (const dbl_t* t : k.keep)
@@ -897,7 +916,7 @@ struct PlanKeyHash
     }
 };
 std::unordered_map<PlanKey, Plan, PlanKeyHash> g_plans;
-std::unordered_set<const dbl_t*> g_keep;
+Keep g_keep;
 
 }  // namespace
 
@@ -937,8 +956,15 @@ void synchronize()
 
 void set_protected_tensors(const std::vector<const dbl_t*>& tensors)
 {
-    g_keep.clear();
-    g_keep.insert(tensors.begin(), tensors.end());
+    g_keep.all = false;
+    g_keep.set.clear();
+    g_keep.set.insert(tensors.begin(), tensors.end());
+}
+
+void protect_all_tensors()
+{
+    g_keep.all = true;
+    g_keep.set.clear();
 }
 
 // ---- inputs fed from host memory --------------------------------------------------------------
@@ -1010,9 +1036,16 @@ void feed(dbl_t* dst, const dbl_t* src_host, std::size_t count)
     g_feeds.push_back(Feed{dst, dst + count, src_host});
 }
 
+void drop_feeds()
+{
+    g_feeds.clear();
+}
+
 void run_async(rt::NodesList& tasks)
 {
-    PlanKey key{tasks.nodes(), std::vector<const dbl_t*>(g_keep.begin(), g_keep.end()), fusion()};
+    // the inputs noted for this run are borrowed host buffers: whatever happens, none outlives it
+    struct DropFeeds { ~DropFeeds() { g_feeds.clear(); } } drop_feeds_on_exit;
+    PlanKey key{tasks.nodes(), std::vector<const dbl_t*>(g_keep.set.begin(), g_keep.set.end()), g_keep.all, fusion()};
     std::sort(key.keep.begin(), key.keep.end());
     auto it = g_plans.find(key);
     if (it == g_plans.end())
@@ -1050,36 +1083,3 @@ void forget_plans()
 }
 
 }  // namespace hip
-
-namespace rt
-{
-namespace
-{
-runner_f g_cpu[2] = {nullptr, nullptr};
-}
-
-void register_cpu_backend(ProgramMode mode, runner_f runner)
-{
-    if (mode == ProgramMode::MONOTHREAD) g_cpu[0] = runner;
-    if (mode == ProgramMode::MULTITHREAD) g_cpu[1] = runner;
-}
-
-void execute(NodesList& tasks)
-{
-    const ProgramMode mode = program_mode();
-    if (mode == ProgramMode::GPU)
-    {
-        if (hip::sync_each_run())
-            hip::run(tasks);
-        else
-            hip::run_async(tasks);
-        return;
-    }
-    runner_f r = g_cpu[mode == ProgramMode::MONOTHREAD ? 0 : 1];
-    if (!r)
-        throw std::runtime_error(
-            "RT_MODE selects a CPU mode, but this library only holds the HIP backend (RT_MODE=GPU); "
-            "the CPU runners are the reference's src/cpu tree -- register one with rt::register_cpu_backend");
-    r(tasks);
-}
-}  // namespace rt

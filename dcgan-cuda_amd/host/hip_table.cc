@@ -21,6 +21,13 @@ void check(int rc, const char* what)
 
 #define CK(call) check((call), #call)
 
+const char* op_name(int type)
+{
+    if (type == rt::Node::OP_NOP)
+        return "nop";
+    return type >= 0 && type <= rt::Node::OP_ADD ? rt::Node::OP_NAMES[type] : "?";
+}
+
 
 // conv2d forward.  Node fields: src/runtime/node.cu:118-141; decode: src/gpu/conv2d.cu:13-40.
 ConvGeom geom_conv2d(const rt::Node* n)

@@ -44,6 +44,9 @@ ConvGeom geom_transpose(const rt::Node* n);
 ConvGeom geom_transpose_input_grad(const rt::Node* n);
 ConvGeom geom_transpose_kernel_grad(const rt::Node* n);
 
+// The operator's name as rt::Node::OP_NAMES spells it ("nop" for the placeholder, "?" outside the table).
+const char* op_name(int type);
+
 // Advances the host-side step counter of an adam_update node (node->out2) and returns the
 // bias-corrected rate, formed in float exactly as src/gpu/update.cu:81-93 does.
 float adam_advance(rt::Node* n);

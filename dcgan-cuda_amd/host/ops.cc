@@ -237,54 +237,67 @@ void Graph::run(std::vector<Op*> ops, const std::map<Input*, std::pair<const dbl
             targets.push_back(c.out_node);
     }
 
-    for (const auto& kv : inputs)
+    // From the first input noted to the end of the run the backend holds borrowed host pointers: an
+    // exception on the way (an operator that cannot be lowered, a cycle, a failing launch) drops them.
+    try
     {
-        compile_(kv.first);
-        dbl_t* dst = compiled(kv.first).out_data;
-        // DCGAN_HIP_FEED=front: the copy in front of the run, as the reference places it
-        static const bool deferred = !(std::getenv("DCGAN_HIP_FEED") && !std::strcmp(std::getenv("DCGAN_HIP_FEED"), "front"));
-        if (program_mode() == ProgramMode::GPU && deferred)
-            hip::feed(dst, kv.second.first, (std::size_t)kv.second.second.total());
+        for (const auto& kv : inputs)
+        {
+            compile_(kv.first);
+            dbl_t* dst = compiled(kv.first).out_data;
+            // DCGAN_HIP_FEED=front: the copy in front of the run, as the reference places it
+            static const bool deferred = !(std::getenv("DCGAN_HIP_FEED") && !std::strcmp(std::getenv("DCGAN_HIP_FEED"), "front"));
+            if (program_mode() == ProgramMode::GPU && deferred)
+                hip::feed(dst, kv.second.first, (std::size_t)kv.second.second.total());
+            else
+                tensor_write(dst, dst + kv.second.second.total(), kv.second.first);
+        }
+
+        // the execution order depends only on the requested operators: computed once, then reused
+        auto sched = schedules_.find(ops);
+        if (sched == schedules_.end())
+            sched = schedules_.emplace(ops, full_rt_graph_->topological_sort(targets)).first;
+        last_schedule_ = sched->second;
+        rt::NodesList list(sched->second);
+        if (debug_)
+        {
+            const ProgramMode m = program_mode();
+            std::cout << "run program in "
+                      << (m == ProgramMode::GPU ? "gpu" : m == ProgramMode::MULTITHREAD ? "multithread" : "monothread")
+                      << "\n" << list;
+        }
+
+        std::vector<const dbl_t*> wanted;
+        for (std::size_t i = 0; i < outputs.size() && i < ops.size(); ++i)
+            if (outputs[i])
+                wanted.push_back(compiled(ops[i]).out_data);
+        if (name_results_)
+            hip::set_protected_tensors(wanted);
         else
-            tensor_write(dst, dst + kv.second.second.total(), kv.second.first);
-    }
-
-    // the execution order depends only on the requested operators: computed once, then reused
-    auto sched = schedules_.find(ops);
-    if (sched == schedules_.end())
-        sched = schedules_.emplace(ops, full_rt_graph_->topological_sort(targets)).first;
-    last_schedule_ = sched->second;
-    rt::NodesList list(sched->second);
-    if (debug_)
-    {
-        const ProgramMode m = program_mode();
-        std::cout << "run program in "
-                  << (m == ProgramMode::GPU ? "gpu" : m == ProgramMode::MULTITHREAD ? "multithread" : "monothread")
-                  << "\n" << list;
-    }
-
-    std::vector<const dbl_t*> wanted;
-    for (std::size_t i = 0; i < outputs.size() && i < ops.size(); ++i)
-        if (outputs[i])
-            wanted.push_back(compiled(ops[i]).out_data);
-    hip::set_protected_tensors(wanted);
-    if (!wanted.empty() && program_mode() == ProgramMode::GPU && hip::sync_each_run())
-    {
-        // the blocking device-to-host copy of the first result waits for the run: no separate wait
-        hip::set_sync_each_run(false);
-        try
+            hip::protect_all_tensors();
+        if (!wanted.empty() && program_mode() == ProgramMode::GPU && hip::sync_each_run())
         {
-            rt::execute(list);
-        }
-        catch (...)
-        {
+            // the blocking device-to-host copy of the first result waits for the run: no separate wait
+            hip::set_sync_each_run(false);
+            try
+            {
+                rt::execute(list);
+            }
+            catch (...)
+            {
+                hip::set_sync_each_run(true);
+                throw;
+            }
             hip::set_sync_each_run(true);
-            throw;
         }
-        hip::set_sync_each_run(true);
+        else
+            rt::execute(list);
     }
-    else
-        rt::execute(list);
+    catch (...)
+    {
+        hip::drop_feeds();
+        throw;
+    }
 
     for (std::size_t i = 0; i < outputs.size() && i < ops.size(); ++i)
     {

@@ -156,6 +156,10 @@ public:
     Op* gradient(Op* out, Op* var);
 
     void debug_set(bool debug) { debug_ = debug; }
+    // Off: run() hands the backend nothing but the instruction list, as src/ops/graph.cu:194-200 does
+    // (hip::protect_all_tensors: every intermediate result is kept).  On (default): run() names the
+    // tensors it reads back (hip::set_protected_tensors) and the backend may leave the others out.
+    void name_results_set(bool on) { name_results_ = on; }
     // Trainable variables, in creation order, to / from a file: numpy's .npz when the path ends in
     // ".npz" (arrays arr_0, arr_1, ...), else a `DGV1` header followed per variable by the element
     // count and the fp32 data.
@@ -187,6 +191,7 @@ private:
     std::vector<rt::Node*> last_schedule_;
     rt::Graph* full_rt_graph_ = new rt::Graph;
     bool debug_ = false;
+    bool name_results_ = true;
 };
 
 class OpsBuilder

@@ -32,6 +32,7 @@ def load():
         lib.dg_destroy.argtypes = [C.c_void_p]
         lib.dg_set_fusion.argtypes = [C.c_int]
         lib.dg_set_pairing.argtypes = [C.c_int]
+        lib.dg_set_name_results.argtypes = [C.c_int]
         lib.dg_num_vars.argtypes = [C.c_void_p]
         lib.dg_var_size.argtypes = [C.c_void_p, C.c_int]
         lib.dg_var_size.restype = C.c_long
@@ -112,6 +113,12 @@ class DcganModel:
 
     def set_fusion(self, on):
         self.lib.dg_set_fusion(1 if on else 0)
+
+    def set_name_results(self, on):
+        """Off: a run hands the backend the instruction list and nothing else, as the reference's
+        Graph::run does (src/ops/graph.cu:194-200); every intermediate tensor is then kept.  On (default):
+        the run names the tensors it reads back and the planner may leave out the others."""
+        self.lib.dg_set_name_results(1 if on else 0)
 
     def set_pairing(self, on):
         """With fusion: run same-filter convolutions of the two discriminator towers as one launch."""

@@ -94,8 +94,9 @@ size_t dh_workspace_bytes(void);
  * so a training loop -- and a recompile at another shape that fits what is held -- makes no hipMalloc or
  * hipFree.  A freed block may be handed out again at once: correct for callers that queue all work on one
  * stream (the stream orders the old tensor's last use before the new one's first); others synchronise or
- * order their streams before freeing.  dh_pool_reserve makes sure that at least `bytes` are held and
- * idle, dh_pool_trim returns idle slabs to the driver (after a device synchronisation), dh_pool_stats
+ * order their streams before freeing.  dh_pool_reserve makes sure that ONE idle range of at least
+ * `bytes` is held (a dh_pool_alloc of up to that size that follows makes no hipMalloc, however fragmented the
+ * rest is), dh_pool_trim returns idle slabs to the driver (after a device synchronisation), dh_pool_stats
  * reports hipMalloc calls made so far, bytes held, bytes handed out and their peak (any may be NULL). */
 int dh_pool_alloc(void** ptr, size_t bytes);
 int dh_pool_free(void* ptr);
@@ -213,7 +214,8 @@ int dh_bias_grad_parts(const float* dz, float* parts, size_t rows, size_t cols, 
  * dh_bias_grad_part_count(rows, cols) * cols floats exceed the buffer.  Every call on a GPU shares
  * that GPU's buffer (each range sum is written before it is read, so nothing needs clearing): calls
  * that overlap on one GPU -- from different streams or threads -- race; calls on one stream are
- * ordered by the stream. */
+ * ordered by the stream.  dh_init must have run on the device before a stream capture begins: the first
+ * library call on a device otherwise initialises it (and looks the buffer's address up) inside that call. */
 int dh_bias_grad_static(const float* dz, float* db, size_t rows, size_t cols, void* stream);
 size_t dh_bias_grad_static_max_bytes(void);
 /* out[r] = sum_c a[r,c].  Replaces gpu::mat_sum_rows (src/gpu/sum.cu:69-108). */

@@ -8,6 +8,13 @@
 // runs them through hip::kernels_list[node->type] on device buffers and through
 // cpu::kernels_list[node->type] on host buffers, and compares (src/gpu/kernels.cu:23-61,
 // src/gpu/runner.cu:10-18 are what hip_table.cc replaces).
+//
+// The planning runner, dcgan-cuda_amd/host/hip_kernels.cc, is compiled into the same library the same
+// way -- unchanged, against the reference's node.hh and nodes-list.hh.  The seam_prog_* calls build a
+// whole instruction graph in the reference's rt::Graph (src/runtime/graph.cu), order it with the
+// reference's rt::Graph::topological_sort as src/ops/graph.cu:194-200 does, and run the resulting
+// rt::NodesList through hip::run (fused and paired launches) or, node by node, through the reference's
+// CPU table.
 #include <cstddef>
 #include <cstring>
 #include <exception>
@@ -15,14 +22,26 @@
 #include <vector>
 
 #include "cpu/kernels.hh"
+#include "runtime/graph.hh"
 #include "runtime/node.hh"
+#include "runtime/nodes-list.hh"
 
+#include "hip_runner.hh"
 #include "hip_table.hh"
 
 namespace
 {
 std::string g_error;
 }
+
+// An instruction graph owned by the reference's rt::Graph; nodes are addressed by creation order.
+struct Prog
+{
+    rt::Graph graph;
+    std::vector<rt::Node*> nodes;
+};
+
+rt::Node* make_node(const char* op, float** t, const int* i, const float* f, const std::vector<rt::Node*>& preds);
 
 extern "C" {
 
@@ -55,8 +74,13 @@ int seam_node_layout(unsigned long* out, int n)
 // flattened); f[]: the float arguments in the factory's order.  Returns NULL for an unknown name.
 void* seam_node_new(const char* op, float** t, const int* i, const float* f)
 {
+    return make_node(op, t, i, f, {});
+}
+}  // extern "C"
+
+rt::Node* make_node(const char* op, float** t, const int* i, const float* f, const std::vector<rt::Node*>& none)
+{
     const std::string o(op);
-    const std::vector<rt::Node*> none;
     using N = rt::Node;
     if (o == "conv2d") return N::op_conv2d(t[0], t[1], i, i[2], i[3], t[3], i + 4, i + 8, none);
     if (o == "conv2d_input_grad") return N::op_conv2d_input_grad(t[0], t[1], i, t[3], i + 2, i + 6, i + 10, none);
@@ -95,6 +119,8 @@ void* seam_node_new(const char* op, float** t, const int* i, const float* f)
     return nullptr;
 }
 
+extern "C" {
+
 int seam_node_type(void* node) { return static_cast<rt::Node*>(node)->type; }
 void seam_node_free(void* node) { delete static_cast<rt::Node*>(node); }
 
@@ -132,4 +158,101 @@ int seam_run_hip(void* node)
 // 1 where the HIP table has an entry for the op code, 0 where it is nullptr.
 int seam_hip_has(int type) { return type >= 0 && type < 512 && hip::kernels_list[type] != nullptr; }
 int seam_cpu_has(int type) { return type >= 0 && type < 512 && cpu::kernels_list[type] != nullptr; }
+
+// ---- whole instruction graphs through the planning runner ----------------------------------------
+void* seam_prog_new(void) { return new Prog(); }
+void seam_prog_free(void* prog) { delete static_cast<Prog*>(prog); }   // rt::Graph deletes its nodes
+
+// Adds one instruction made by the reference's factory `op` (arguments as for seam_node_new) whose
+// predecessors are the instructions pred[0..npred), given by their ids; returns the new id, -1 for
+// an unknown factory.
+int seam_prog_add(void* prog, const char* op, float** t, const int* i, const float* f, const int* pred, int npred)
+{
+    Prog* p = static_cast<Prog*>(prog);
+    std::vector<rt::Node*> preds;
+    for (int q = 0; q < npred; ++q)
+        preds.push_back(p->nodes.at((std::size_t)pred[q]));
+    rt::Node* n = make_node(op, t, i, f, preds);
+    if (!n)
+        return -1;
+    p->graph.add(n);
+    p->nodes.push_back(n);
+    return (int)p->nodes.size() - 1;
+}
+
+// The order the reference would execute in for the requested instructions (src/ops/graph.cu:196):
+// writes up to `cap` ids, returns the length of the list.
+int seam_prog_order(void* prog, const int* want, int nwant, int* ids, int cap)
+{
+    Prog* p = static_cast<Prog*>(prog);
+    std::vector<rt::Node*> targets;
+    for (int q = 0; q < nwant; ++q)
+        targets.push_back(p->nodes.at((std::size_t)want[q]));
+    rt::NodesList list(p->graph.topological_sort(targets));
+    int n = 0;
+    for (rt::Node* node : list.nodes())
+    {
+        for (std::size_t id = 0; id < p->nodes.size(); ++id)
+            if (p->nodes[id] == node && n < cap)
+                ids[n] = (int)id;
+        ++n;
+    }
+    return n;
+}
+
+// Runs the sorted list node by node through the reference's CPU table (cpu::run_sequential without its
+// debug output, src/cpu/runner.cu).
+int seam_prog_run_cpu(void* prog, const int* want, int nwant)
+{
+    Prog* p = static_cast<Prog*>(prog);
+    try
+    {
+        std::vector<rt::Node*> targets;
+        for (int q = 0; q < nwant; ++q)
+            targets.push_back(p->nodes.at((std::size_t)want[q]));
+        rt::NodesList list(p->graph.topological_sort(targets));
+        for (rt::Node* n : list.nodes())
+            cpu::kernels_list[n->type](n);
+        return 0;
+    }
+    catch (const std::exception& e)
+    {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+// Runs the sorted list through hip::run.  fuse / pair: the planner's switches.  nkeep < 0: the caller
+// names no tensors, as gpu::run's signature has it (every tensor is then kept); otherwise
+// keep[0..nkeep) go to hip::set_protected_tensors first, the one call a fused drop-in adds to
+// src/ops/graph.cu.  *launches receives the number of steps the plan issued.
+int seam_prog_run_hip(void* prog, const int* want, int nwant, int fuse, int pair, float** keep, int nkeep, int* launches)
+{
+    Prog* p = static_cast<Prog*>(prog);
+    try
+    {
+        std::vector<rt::Node*> targets;
+        for (int q = 0; q < nwant; ++q)
+            targets.push_back(p->nodes.at((std::size_t)want[q]));
+        rt::NodesList list(p->graph.topological_sort(targets));
+        hip::set_fusion(fuse != 0);
+        hip::set_pairing(pair != 0);
+        hip::forget_plans();
+        if (nkeep < 0)
+            hip::protect_all_tensors();
+        else
+            hip::set_protected_tensors(std::vector<const dbl_t*>(keep, keep + nkeep));
+        hip::run(list);
+        if (launches)
+            *launches = hip::last_launch_count();
+        hip::forget_plans();
+        hip::protect_all_tensors();
+        return 0;
+    }
+    catch (const std::exception& e)
+    {
+        g_error = e.what();
+        return 1;
+    }
+}
 }

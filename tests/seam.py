@@ -74,3 +74,69 @@ def run_both(A, op, arrays, ints=(), floats=(), host_slots=()):
         lib.seam_node_free(n)
     got = [None if a is None else (a if s in host_slots else dev[s].numpy()) for s, a in enumerate(host)]
     return (cpu[3], cpu[4]), (got[3], got[4]), code
+
+
+class Program:
+    """An instruction graph held by the REFERENCE's rt::Graph (src/runtime/graph.cu): instructions come
+    from the reference's factories with explicit predecessors, the execution order from the reference's
+    topological_sort, and the list runs through the reference's CPU table or through hip::run -- the
+    planning runner compiled against the reference's node.hh / nodes-list.hh."""
+
+    def __init__(self):
+        lib = load()
+        lib.seam_prog_new.restype = C.c_void_p
+        lib.seam_prog_free.argtypes = [C.c_void_p]
+        lib.seam_prog_add.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_int),
+                                      C.POINTER(C.c_float), C.POINTER(C.c_int), C.c_int]
+        lib.seam_prog_order.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.POINTER(C.c_int), C.c_int]
+        lib.seam_prog_run_cpu.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int]
+        lib.seam_prog_run_hip.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_int, C.c_int,
+                                          C.POINTER(C.c_void_p), C.c_int, C.POINTER(C.c_int)]
+        self.lib = lib
+        self.h = C.c_void_p(lib.seam_prog_new())
+        self.count = 0
+
+    def close(self):
+        if self.h:
+            self.lib.seam_prog_free(self.h)
+            self.h = None
+
+    def add(self, op, tensors, ints=(), floats=(), preds=()):
+        """tensors: five addresses as for node(); preds: ids of the instructions this one waits for."""
+        t = (C.c_void_p * 5)(*[C.c_void_p(int(a)) if a else None for a in tensors])
+        i = (C.c_int * max(len(ints), 1))(*[int(v) for v in ints])
+        f = (C.c_float * max(len(floats), 1))(*[float(v) for v in floats])
+        p = (C.c_int * max(len(preds), 1))(*[int(v) for v in preds])
+        nid = self.lib.seam_prog_add(self.h, op.encode(), t, i, f, p, len(preds))
+        if nid < 0:
+            raise KeyError("no reference factory bound for " + op)
+        self.count += 1
+        return nid
+
+    @staticmethod
+    def _ids(want):
+        return (C.c_int * max(len(want), 1))(*[int(v) for v in want]), len(want)
+
+    def order(self, want):
+        w, n = self._ids(want)
+        ids = (C.c_int * (self.count + 1))()
+        got = self.lib.seam_prog_order(self.h, w, n, ids, self.count + 1)
+        return list(ids)[:got]
+
+    def run_cpu(self, want):
+        w, n = self._ids(want)
+        if self.lib.seam_prog_run_cpu(self.h, w, n) != 0:
+            raise RuntimeError(self.lib.seam_last_error().decode())
+
+    def run_hip(self, want, fuse=True, pair=True, keep=None):
+        """keep=None: nothing is said about the tensors read afterwards (gpu::run's own signature);
+        otherwise the addresses handed to hip::set_protected_tensors.  Returns the launch count."""
+        w, n = self._ids(want)
+        launches = C.c_int(0)
+        if keep is None:
+            k, nk = (C.c_void_p * 1)(), -1
+        else:
+            k, nk = (C.c_void_p * max(len(keep), 1))(*[C.c_void_p(int(a)) for a in keep]), len(keep)
+        if self.lib.seam_prog_run_hip(self.h, w, n, int(fuse), int(pair), k, nk, C.byref(launches)) != 0:
+            raise RuntimeError(self.lib.seam_last_error().decode())
+        return launches.value

@@ -49,14 +49,17 @@ def cpu_dump64_f64(tmp_path_factory):
 
 def gpu_dump(fusion, batch=BATCH, steps=1, one_run=False, tile=1):
     """fusion: False (one launch per instruction), True (fused launches, the two discriminator towers'
-    convolutions paired), "unpaired" (fused launches, every convolution on its own).  tile > 1: the
-    model runs at tile * batch with the batch's inputs repeated tile times."""
+    convolutions paired), "unpaired" (fused launches, every convolution on its own), "list only" (the
+    planner is handed the instruction list and nothing else, as the reference's Graph::run calls gpu::run,
+    and makes only the fusions that keep every tensor).  tile > 1: the model runs at tile * batch with
+    the batch's inputs repeated tile times."""
     import __graft_entry__ as ge
     pkg = ge.load_package()
     model = pkg.hostabi.DcganModel(batch * tile, SEED, "GPU")
     try:
         model.set_fusion(bool(fusion))
         model.set_pairing(fusion != "unpaired")
+        model.set_name_results(fusion != "list only")
         w, z, x = dr.synthetic(batch, SEED, pkg.hostabi.var_shapes())
         for name, val in w.items():
             model.set_var(name, val)
@@ -65,6 +68,7 @@ def gpu_dump(fusion, batch=BATCH, steps=1, one_run=False, tile=1):
     finally:
         model.set_fusion(False)
         model.set_pairing(True)
+        model.set_name_results(True)
         model.close()
 
 
@@ -148,7 +152,7 @@ def agree_with_yardstick(key, got, exp32, exp64, kinks=0):
         assert frac <= 2.0 * frac32 + 1e-4, "%s: %.3g of the elements moved differently (oracle fp32: %.3g)" % (key, frac, frac32)
 
 
-@pytest.mark.parametrize("fusion", [True, False])
+@pytest.mark.parametrize("fusion", [True, False, "list only"])
 def test_training_iterations_at_batch_64(cpu_dump64, cpu_dump64_f64, fusion):
     """The benchmarked configuration: every layer of both networks, the four losses, all 21 gradients
     (one run of the graph for all of them), then three training iterations (D step, G step; with

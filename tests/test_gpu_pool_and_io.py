@@ -66,6 +66,33 @@ def test_pool_blocks_are_aligned_reused_and_merged(pkg):
         A.check(lib.dh_pool_free(c))
 
 
+def test_a_reservation_is_one_range_not_a_sum_of_fragments(pkg):
+    """Idle fragments that add up to the reserved size do not count: after dh_pool_reserve(n) a block of n
+    bytes is served without a hipMalloc."""
+    A = pkg.hipabi
+    lib = A.load()
+    import ctypes as C
+
+    def alloc(n):
+        p = C.c_void_p()
+        A.check(lib.dh_pool_alloc(C.byref(p), n))
+        return p.value
+
+    mib = 1 << 20
+    blocks = [alloc(2 * mib) for _ in range(8)]
+    for b in blocks[::2]:              # every other block back: 8 MiB idle in pieces of 2 MiB (plus what was idle before)
+        A.check(lib.dh_pool_free(b))
+    big = 700 * mib                    # larger than any range a batch-64 model leaves idle
+    A.check(lib.dh_pool_reserve(big))
+    before = A.pool_stats()
+    assert before["held"] - before["in_use"] >= big
+    p = alloc(big)
+    assert A.pool_stats()["hipmallocs"] == before["hipmallocs"]
+    for b in blocks[1::2] + [p]:
+        A.check(lib.dh_pool_free(b))
+    A.check(lib.dh_pool_trim())
+
+
 def test_training_loop_and_a_rebuild_at_another_batch_allocate_nothing(pkg):
     """After the first iteration neither the tensor pool nor the scratch arenas grow; a model torn down
     and built again at a smaller batch (every operator lowered anew, at other shapes) is served from the

@@ -14,9 +14,10 @@ def both(A, lib, dz):
     ref, got = A.Buf((cols,)), A.Buf((cols,))
     A.check(lib.dh_memset0(got.ptr, cols * 4, None))
     A.check(lib.dh_bias_grad(d.ptr, ref.ptr, rows, cols, None))
-    before = lib.dh_workspace_bytes()
+    before, pool = lib.dh_workspace_bytes(), A.pool_stats()
     A.check(lib.dh_bias_grad_static(d.ptr, got.ptr, rows, cols, None))
     assert lib.dh_workspace_bytes() == before
+    assert A.pool_stats() == pool           # no hipMalloc, no block handed out by the tensor pool either
     return ref.numpy(), got.numpy()
 
 
