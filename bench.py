@@ -18,6 +18,8 @@ Prints ONE JSON line.  Besides the contract fields it carries
 gradient separately; BASELINE.json config 1) at `--batch`, each timed over a sustained run, and
 prints one JSON line with a row per (layer, operator).  `--workload generator --batch 4096` times
 the generator's forward pass alone (BASELINE.json config 4's inference half; config 0 at batch 64).
+`--workload discriminator` times the discriminator's forward and backward pass on labelled images
+(BASELINE.json config 2: all dW / db and the gradient of the images, no optimiser).
 `cpu_baseline.mcpu` is the reference's RT_MODE=MCPU runtime (4 workers) on the same sample.
 `--workload streaming` times the memory-bound operators (bias, activations, their gradients, Adam)
 on 128 MiB tensors, as algorithmic GB/s against the HBM peak, with a plain copy beside them.
@@ -441,6 +443,87 @@ def generator_only(args, pkg, A):
     model.close()
 
 
+def discriminator_pass(args, pkg, A):
+    """BASELINE.json config 2: the discriminator forward and backward on labelled images (random 0/1 labels) --
+    four convolutions with bias and leaky relu, the dense head, sigmoid cross-entropy, and the gradients of all
+    ten variables and of the input images, no optimiser (tests/test_dcgan_discriminator.cu:49-136 at batch 64).
+    Images and labels are resident, nothing is read back; one step = one pass over the batch."""
+    weights, _, x = synthetic(args.batch)
+    y = (np.random.default_rng(99).random((args.batch, 1)) < 0.5).astype(np.float32)
+    model = pkg.hostabi.DcganModel(args.batch, seed=1, mode="GPU")
+    model.set_fusion(bool(args.fusion))
+    for name, w in weights.items():
+        model.set_var(name, w)
+    model.set_inputs(x=x)
+    model.set_labels(y)
+    for _ in range(args.warmup):
+        model.disc_pass(want_loss=False)
+    model.sync()
+    launches = model.last_launch_count()
+    A.profile_reset()
+    every = max(1, args.profile_every)
+    timer = A.Timer()
+    t0 = time.perf_counter()
+    timer.start()
+    profiled = 0
+    for i in range(args.steps):
+        on = i % every == 0
+        if on:
+            A.profile_enable(1)
+            profiled += 1
+        model.disc_pass(want_loss=False)
+        if on:
+            A.profile_enable(0)
+    gpu_ms = timer.stop_ms()
+    model.sync()
+    wall = time.perf_counter() - t0
+    rows = A.profile_read()
+    A.profile_reset()
+    A.profile_enable(2)
+    aux_steps = max(1, min(20, args.steps))
+    for _ in range(aux_steps):
+        model.disc_pass(want_loss=False)
+    model.sync()
+    A.profile_enable(False)
+    aux_rows = A.profile_read()
+    loss = model.disc_pass()
+    # forward, filter gradient and input gradient of all four layers (the images' gradient included) + dense head
+    flops = 3 * sum(conv_flops(args.batch, l) for l in LAYERS) + 3 * 2.0 * args.batch * 8192
+    conv_ms = sum(r["ms"] for r in rows)
+    conv_fl = sum(r["flops"] for r in rows)
+    dom = max(rows, key=lambda r: r["ms"])
+    achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+    hbm_rows = [r for r in aux_rows if r["name"].startswith("hbm:")]
+    print(json.dumps({
+        "metric": "DCGAN discriminator forward+backward passes/sec, fp32", "value": round(args.steps / wall, 2),
+        "unit": "passes/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[2]: DCGAN discriminator forward + backward, fp32, batch %d, images [%d,64,64,3] "
+                               "~ U(-1,1), random 0/1 labels, gradients of all weights and of the images"
+                               % (args.batch, args.batch), "batch": args.batch, "fusion": bool(args.fusion)},
+        "gpu_ms_per_step": round(gpu_ms / args.steps, 4), "launches_per_step": launches, "loss": float(loss),
+        "step_gflop": round(flops / 1e9, 2), "step_tflops": round(flops / (wall / args.steps) / 1e12, 3),
+        "images_per_s": round(args.batch * args.steps / wall, 1),
+        "device": A.device_info(),
+        "roofline": {"kernel": dom["name"], "bound": "mfma", "achieved": round(achieved, 3),
+                     "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                     "all_conv_kernels": {"tflops": round(conv_fl / (conv_ms * 1e-3) / 1e12, 3),
+                                          "frac": round(conv_fl / (conv_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                                          "ms_per_step": round(conv_ms / max(profiled, 1), 4)},
+                     "kernels": [{"name": r["name"], "launches": r["launches"],
+                                  "avg_us": round(r["ms"] * 1e3 / r["launches"], 2),
+                                  "tflops": round(r["flops"] / (r["ms"] * 1e-3) / 1e12, 2),
+                                  "frac": round(r["flops"] / (r["ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                                  "issued_frac": round(r["issued"] / (r["ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)
+                                  if r["issued"] > 0 else None}
+                                 for r in sorted(rows, key=lambda r: -r["ms"])],
+                     "hbm_kernels": [hbm_row(r, aux_steps) for r in sorted(hbm_rows, key=lambda r: -r["ms"])]},
+    }))
+    model.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -448,7 +531,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--fusion", type=int, default=1)
-    ap.add_argument("--workload", choices=["iteration", "layers", "generator", "streaming"], default="iteration")
+    ap.add_argument("--workload", choices=["iteration", "layers", "generator", "discriminator", "streaming"], default="iteration")
     ap.add_argument("--elements", type=int, default=1 << 25, help="floats per tensor of --workload streaming")
     ap.add_argument("--sustain-ms", type=float, default=100.0,
                     help="--workload streaming: time each operator over at least this long a run of launches")
@@ -469,6 +552,9 @@ def main():
         return
     if args.workload == "generator":
         generator_only(args, pkg, A)
+        return
+    if args.workload == "discriminator":
+        discriminator_pass(args, pkg, A)
         return
     if args.workload == "streaming":
         streaming_sweep(args, A)

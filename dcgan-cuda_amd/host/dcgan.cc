@@ -134,6 +134,8 @@ Model* build(int batch, unsigned long long seed)
     m.d_fake_loss = builder.sigmoid_cross_entropy(m.labels0, fake_logits);
     m.d_real_loss = builder.sigmoid_cross_entropy(m.labels1, real_logits);
     m.d_loss = builder.add(m.d_fake_loss, m.d_real_loss);
+    m.y = builder.input(ops::Shape({batch, 1}));
+    m.disc_loss = builder.sigmoid_cross_entropy(m.y, real_logits);
 
     for (auto& l : m.g_layers)
     {
@@ -213,6 +215,7 @@ ops::Op* lookup(dcgan::Model& m, const std::string& what)
     if (what == "d_loss") return m.d_loss;
     if (what == "d_fake_loss") return m.d_fake_loss;
     if (what == "d_real_loss") return m.d_real_loss;
+    if (what == "disc_loss") return m.disc_loss;
     if (what.rfind("g_l", 0) == 0)
     {
         const int i = std::stoi(what.substr(3));
@@ -224,11 +227,13 @@ ops::Op* lookup(dcgan::Model& m, const std::string& what)
     {
         const std::size_t c = what.find(':', 5);
         const std::string loss = what.substr(5, c - 5), target = what.substr(c + 1);
-        ops::Op* l = loss == "g_loss" ? m.g_loss : loss == "d_loss" ? m.d_loss : nullptr;
+        ops::Op* l = loss == "g_loss" ? m.g_loss : loss == "d_loss" ? m.d_loss : loss == "disc_loss" ? m.disc_loss : nullptr;
         if (!l)
             throw std::runtime_error("unknown loss " + loss);
         if (target == "x_fake")
             return g.gradient(l, m.g_out);
+        if (target == "x_real")
+            return g.gradient(l, m.x);
         return g.gradient(l, var_at(m, std::stoi(target)));
     }
     throw std::runtime_error("unknown tensor " + what);
@@ -348,6 +353,34 @@ int dg_g_step_fed(void* model, const float* z_host, float* g_loss)
         dcgan::Model& m = M(model);
         hip::set_sync_each_run(g_loss != nullptr);
         ops::Graph::instance().run({m.g_opti, m.g_loss}, fed(m, z_host, nullptr), {nullptr, g_loss});
+        hip::set_sync_each_run(true);
+    });
+}
+
+int dg_set_labels(void* model, const float* y_host)
+{
+    return guarded([&] {
+        dcgan::Model& m = M(model);
+        ops::Graph::instance().run({m.y}, {{m.y, {y_host, ops::Shape({m.batch, 1})}}}, {});
+    });
+}
+
+int dg_disc_pass(void* model, float* loss)
+{
+    return guarded([&] {
+        dcgan::Model& m = M(model);
+        auto& g = ops::Graph::instance();
+        if (m.disc_targets.empty())
+        {
+            m.disc_targets.push_back(m.disc_loss);
+            for (ops::Variable* v : m.d_vars)
+                m.disc_targets.push_back(g.gradient(m.disc_loss, v));
+            m.disc_targets.push_back(g.gradient(m.disc_loss, m.x));
+        }
+        std::vector<dbl_t*> outs(m.disc_targets.size(), nullptr);
+        outs[0] = loss;
+        hip::set_sync_each_run(loss != nullptr);
+        g.run(m.disc_targets, {}, outs);
         hip::set_sync_each_run(true);
     });
 }

@@ -31,6 +31,12 @@ struct Model
     std::vector<ops::Variable*> g_vars, d_vars;        // (w, b) per layer, dense last -- dcgan/main.cu:309-325
     ops::Op *g_opti = nullptr, *d_opti = nullptr;
     std::vector<dbl_t> ones, zeros;
+    // The discriminator by itself on labelled images (tests/test_dcgan_discriminator.cu:49-136): labels y,
+    // loss = sigmoid cross-entropy(y, D(x)) on the tower fed by x, and the pass's targets -- the loss, its
+    // gradient for every discriminator variable and for the images themselves.
+    ops::Input* y = nullptr;
+    ops::Op* disc_loss = nullptr;
+    std::vector<ops::Op*> disc_targets;
 };
 
 // Builds the whole graph (both networks, losses, gradients, Adam).  Weights ~ N(0, 0.02) from
@@ -49,6 +55,11 @@ void dg_destroy(void* model);
 void dg_set_fusion(int fuse);
 // on != 0 (the default): with fusion, same-filter convolutions of independent towers run as one paired launch.
 void dg_set_pairing(int on);
+// The discriminator alone (forward + backward, no optimiser): dg_set_labels binds the [batch, 1] labels,
+// dg_disc_pass computes the loss, all ten parameter gradients and the gradient of the input images in one run
+// (loss == NULL: nothing is read back and the run is not waited for).
+int dg_set_labels(void* model, const float* y_host);
+int dg_disc_pass(void* model, float* loss);
 // on == 0: every run hands the backend its instruction list and nothing else, as the reference's Graph::run
 // does (src/ops/graph.cu:194-200), so the planner keeps every intermediate tensor; on != 0 (the default): the
 // run names the tensors it reads back and the others may be left out.

@@ -33,6 +33,8 @@ def load():
         lib.dg_set_fusion.argtypes = [C.c_int]
         lib.dg_set_pairing.argtypes = [C.c_int]
         lib.dg_set_name_results.argtypes = [C.c_int]
+        lib.dg_set_labels.argtypes = [C.c_void_p, _fp]
+        lib.dg_disc_pass.argtypes = [C.c_void_p, _fp]
         lib.dg_num_vars.argtypes = [C.c_void_p]
         lib.dg_var_size.argtypes = [C.c_void_p, C.c_int]
         lib.dg_var_size.restype = C.c_long
@@ -159,6 +161,20 @@ class DcganModel:
         _check(self.lib.dg_g_step_fed(self.h, None if z is None else _p(z), C.byref(loss) if want_loss else None))
         return loss.value if want_loss else None
 
+    def set_labels(self, y):
+        """Labels [batch, 1] of the stand-alone discriminator pass."""
+        y = np.ascontiguousarray(y, np.float32)
+        assert y.size == self.batch
+        _check(self.lib.dg_set_labels(self.h, _p(y)))
+
+    def disc_pass(self, want_loss=True):
+        """The discriminator alone on the resident images and labels: loss, the gradients of all ten
+        discriminator variables and of the images, one run (names: disc_loss, grad:disc_loss:<var>,
+        grad:disc_loss:x_real)."""
+        loss = C.c_float()
+        _check(self.lib.dg_disc_pass(self.h, C.byref(loss) if want_loss else None))
+        return loss.value if want_loss else None
+
     def sync(self):
         _check(self.lib.dg_sync())
 
@@ -191,7 +207,7 @@ class DcganModel:
 
     @staticmethod
     def grad_name(loss, name):
-        return "grad:%s:%s" % (loss, "x_fake" if name == "x_fake" else VAR_NAMES.index(name))
+        return "grad:%s:%s" % (loss, name if name in ("x_fake", "x_real") else VAR_NAMES.index(name))
 
     def grad(self, loss, name):
         if name == "x_fake":

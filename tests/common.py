@@ -10,7 +10,7 @@ import numpy as np
 RTOL, ATOL = 1e-4, 1e-5
 
 
-def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
+def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=0, kink_extra=0.0):
     """The two-sided parity check of the batch-64 suites.  `exp32` is the oracle's fp32 result (the
     reference's arithmetic and summation order), `exp64` the same computed with float64 sums.
       * element by element: |got - exp32| <= 1e-4 |exp32| + max(1e-5 max(1, max|exp32|), 3 max|exp32 - exp64|)
@@ -36,10 +36,13 @@ def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
     +4.4e-8 in float64, and entry 16 of that layer's bias gradient, 0.0348, moves by 5.7e-5 = 0.8 times the
     gradient arriving there; the eight entries of that layer's filter gradient that meet the largest inputs
     move by up to 1.35e-5 = 2.3e-3 of the tensor's largest entry).  A caller sets `kinks` only where it has
-    FOUND such an element (the DCGAN tests look for layer outputs of opposite sign at the rounding level).  Such
-    tensors are allowed 5e-3 of their largest magnitude in the float64 check, their relative L2 error is
-    held to 1e-3, and in the element-by-element check one entry (one per 100 000 for larger tensors) may be
-    off by up to that 5e-3 as well."""
+    FOUND such elements, and passes their number (the DCGAN tests look for layer outputs of opposite sign at the
+    rounding level and count those the gradient flows back through).  Such tensors are allowed 5e-3 of their
+    largest magnitude in the float64 check, their relative L2 error is held to 1e-3, and in the
+    element-by-element check one entry per kink (one per 100 000 entries and kink for larger tensors: a flipped
+    slope reaches a whole filter column) may be off by up to that 5e-3 as well.  kink_extra is added to that
+    allowance where the caller can bound the flipped slope's direct effect from the data (the filter gradient of
+    the kinked layer itself moves by input patch x the change of the layer's bias gradient)."""
     got, exp32, exp64 = (np.asarray(a, np.float64).reshape(-1) for a in (got, exp32, exp64))
     mag = float(np.abs(exp32).max()) if exp32.size else 0.0
     yard = float(np.abs(exp32 - exp64).max()) if exp32.size else 0.0
@@ -50,8 +53,8 @@ def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
         atol = max(ATOL * max(1.0, mag), 3.0 * yard)
         over = np.abs(got - exp32) > atol + RTOL * np.abs(exp32)
         # a kink shows in single entries (see above): they are held to the float64 check's 5e-3 instead
-        few = kinks and 0 < int(over.sum()) <= max(1, exp32.size // 100000) and \
-            float(np.abs(got - exp32)[over].max()) <= 5e-3 * mag
+        few = kinks and 0 < int(over.sum()) <= int(kinks) * max(1, exp32.size // 100000) and \
+            float(np.abs(got - exp32)[over].max()) <= 5e-3 * mag + kink_extra
         if few:
             print("%-50s %d entr%s at a kink: off by %.3g" % (what, int(over.sum()), "y" if over.sum() == 1 else "ies",
                                                               float(np.abs(got - exp32)[over].max())), flush=True)
@@ -60,7 +63,7 @@ def agree(got, exp32, exp64, what, slack=1.0, elementwise=True, kinks=False):
     if kinks and exp32.size:
         l2 = float(np.linalg.norm(got - exp64) / max(np.linalg.norm(exp64), 1e-30))
         assert l2 <= 1e-3, "%s: relative L2 error %.3g" % (what, l2)
-    assert err <= max(2.0 * slack * yard, ATOL * min(1.0, mag), 5e-3 * mag if kinks else 0.0), \
+    assert err <= max(2.0 * slack * yard, ATOL * min(1.0, mag), 5e-3 * mag + kink_extra if kinks else 0.0), \
         "%s: max |gpu - f64| = %.3g, the oracle's own fp32 error is %.3g (max |exp| = %.3g)" % (what, err, yard, mag)
 
 

@@ -4,6 +4,7 @@ differentiation, and a script mode that evaluates the network through the host l
 RT_MODE=CPU (the oracle as backend) and dumps everything to an .npz for the GPU parity test.
 
     python tests/dcgan_reference.py <batch> <seed> <out.npz> [<iterations> [f64]]
+    python tests/dcgan_reference.py <batch> <seed> <out.npz> disc [f64]     (the discriminator pass alone)
 """
 import os
 import sys
@@ -29,6 +30,50 @@ def synthetic(batch, seed, shapes):
     z = rng.uniform(-1, 1, (batch, 100)).astype(np.float32)
     x = rng.uniform(-1, 1, (batch, 64, 64, 3)).astype(np.float32)
     return w, z, x
+
+
+def labels(batch, seed):
+    """Random 0/1 labels [batch, 1] of the stand-alone discriminator pass (Bernoulli 1/2)."""
+    return (np.random.default_rng(seed + 1000).random((batch, 1)) < 0.5).astype(np.float32)
+
+
+def disc_names():
+    """(key in the dump, facade name) of the discriminator pass on labelled images, in the manner of
+    tests/test_dcgan_discriminator.cu:49-136: layers, logits, loss, every dW / db, and the gradient of
+    the images."""
+    import __graft_entry__ as ge
+    M = ge.load_package().hostabi.DcganModel
+    names = [("disc_l%d" % i, "d_real_l%d" % i) for i in range(4)] + [("disc_logits", "d_real_logits"), ("disc_loss", "disc_loss")]
+    names += [("grad_disc_loss_" + v, M.grad_name("disc_loss", v)) for v in D_VARS + ["x_real"]]
+    return names
+
+
+def collect_disc(model):
+    """The tensors of disc_names() from ONE run of the graph (weights, images and labels already set)."""
+    names = disc_names()
+    got = model.eval_many([n for _, n in names])
+    return {key: got[n] for key, n in names}
+
+
+def torch_disc(w, x, y):
+    """float64 torch evaluation of the labelled discriminator pass: same keys as collect_disc()."""
+    import torch
+    import torch.nn.functional as F
+    T = {k: torch.tensor(w[k], dtype=torch.float64, requires_grad=True) for k in D_VARS}
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    out, h = {}, xt
+    for i in range(4):
+        ht = F.pad(h.permute(0, 3, 1, 2), (1, 2, 1, 2))
+        h = F.leaky_relu(F.conv2d(ht, T["d%d_w" % i].permute(3, 2, 0, 1), stride=2).permute(0, 2, 3, 1) + T["d%d_b" % i], 0.2)
+        out["disc_l%d" % i] = h
+    logits = h.reshape(x.shape[0], 8192) @ T["d4_w"] + T["d4_b"]
+    out["disc_logits"] = logits
+    out["disc_loss"] = F.binary_cross_entropy_with_logits(logits, torch.tensor(y, dtype=torch.float64))
+    grads = torch.autograd.grad(out["disc_loss"], [T[v] for v in D_VARS] + [xt])
+    res = {k: v.detach().numpy().reshape(-1) for k, v in out.items()}
+    for v, g in zip(D_VARS + ["x_real"], grads):
+        res["grad_disc_loss_" + v] = g.detach().numpy().reshape(-1)
+    return res
 
 
 def tensor_names():
@@ -124,7 +169,8 @@ def torch_dcgan(w, z, x):
 
 def main():
     batch, seed, path = int(sys.argv[1]), int(sys.argv[2]), sys.argv[3]
-    steps = int(sys.argv[4]) if len(sys.argv) > 4 else 1
+    disc = len(sys.argv) > 4 and sys.argv[4] == "disc"
+    steps = int(sys.argv[4]) if len(sys.argv) > 4 and not disc else 1
     import __graft_entry__ as ge
     pkg = ge.load_package()
     f64 = len(sys.argv) > 5 and sys.argv[5] == "f64"
@@ -134,7 +180,11 @@ def main():
     for name, val in w.items():
         model.set_var(name, val)
     model.set_inputs(z, x)
-    np.savez(path, **collect(model, steps))
+    if disc:
+        model.set_labels(labels(batch, seed))
+        np.savez(path, **collect_disc(model))
+    else:
+        np.savez(path, **collect(model, steps))
     model.close()
 
 

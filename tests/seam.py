@@ -76,6 +76,20 @@ def run_both(A, op, arrays, ints=(), floats=(), host_slots=()):
     return (cpu[3], cpu[4]), (got[3], got[4]), code
 
 
+def run_hip(A, op, arrays, ints=(), floats=()):
+    """As run_both, the HIP table only: returns out1 (for shapes where the reference's CPU loops take minutes)."""
+    lib = load()
+    host = [None if a is None else np.array(a, dtype=np.float32, order="C") for a in arrays]
+    dev = [None if a is None else A.Buf.from_numpy(a) for a in host]
+    n = node(op, [0 if d is None else d.ptr for d in dev], ints, floats)
+    try:
+        if lib.seam_run_hip(n) != 0:
+            raise RuntimeError(lib.seam_last_error().decode())
+    finally:
+        lib.seam_node_free(n)
+    return dev[3].numpy()
+
+
 class Program:
     """An instruction graph held by the REFERENCE's rt::Graph (src/runtime/graph.cu): instructions come
     from the reference's factories with explicit predecessors, the execution order from the reference's

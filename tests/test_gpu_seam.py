@@ -43,18 +43,40 @@ CONV_SHAPES = [  # N, H, W, C, kh, kw, O, stride
 
 
 @pytest.mark.parametrize("shape", CONV_SHAPES)
-def test_conv2d_nodes(A, shape):
+def test_conv2d_nodes(A, orc, shape):
     N, H, W, C, kh, kw, O, s = shape
     rng = np.random.default_rng(sum(shape))
     (ph, Ho), (pw, Wo) = same_pad(H, kh, s), same_pad(W, kw, s)
     x, k, dy = rnd(rng, N, H, W, C), rnd(rng, kh, kw, C, O) * 0.1, rnd(rng, N, Ho, Wo, O)
-    small = N < 64      # at the benchmark's size only the forward node: the reference's CPU loops run ~10 s per operator there
+    # At the benchmark's size the reference's CPU loops run ~10 s per forward product and minutes per
+    # gradient: there only the forward node goes through the reference's table; the other nodes -- still made
+    # by the reference's factories and run through the HIP table -- are compared with the oracle, which the
+    # small shapes of this test (and tests/test_oracle_vs_ref.py) tie to the reference's CPU table.
+    small = N < 64
     # conv2d: strides, total pads, input dims, filter dims (src/runtime/node.cu:118-141)
     (e, _), (g, _), code = seam.run_both(A, "conv2d", [x, k, None, np.zeros((N, Ho, Wo, O), np.float32), None],
                                          [s, s, ph, pw, N, H, W, C, kh, kw, C, O])
     assert code == 7
     close(g, e, "conv2d")
     if not small:
+        pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+        g = seam.run_hip(A, "conv2d_input_grad", [dy, k, None, np.zeros((N, H, W, C), np.float32), None],
+                         [s, s, N, Ho, Wo, O, kh, kw, C, O, N, H, W, C])
+        close(g, orc.conv2d_input_grad(dy, k, s, (H, W)), "conv2d_input_grad at batch 64")
+        g = seam.run_hip(A, "conv2d_kernel_grad", [dy, x, None, np.zeros((kh, kw, C, O), np.float32), None],
+                         [s, s, N, Ho, Wo, O, N, H, W, C, ph, pw])
+        close(g, orc.conv2d_kernel_grad(dy, x, s, pads, (kh, kw)), "conv2d_kernel_grad at batch 64")
+        g = seam.run_hip(A, "conv2d_transpose", [dy, k, None, np.zeros((N, H, W, C), np.float32), None],
+                         [N, H, W, C, s, s, N, Ho, Wo, O, kh, kw, C, O])
+        close(g, orc.conv2d_transpose(dy, k, (H, W), s), "conv2d_transpose at batch 64")
+        # gradients of that transpose (x_t := dy, y_t := x): input gradient = conv2d of dy_t, filter gradient
+        # with the roles of the activations exchanged (src/gpu/conv2d.cu:214-307)
+        g = seam.run_hip(A, "conv2d_transpose_input_grad", [x, k, None, np.zeros((N, Ho, Wo, O), np.float32), None],
+                         [s, s, N, H, W, C, kh, kw, C, O, N, Ho, Wo, O])
+        close(g, orc.conv2d_transpose_input_grad(x, k, s, (Ho, Wo)), "conv2d_transpose_input_grad at batch 64")
+        g = seam.run_hip(A, "conv2d_transpose_kernel_grad", [x, dy, None, np.zeros((kh, kw, C, O), np.float32), None],
+                         [s, s, N, H, W, C, N, Ho, Wo, O, kh, kw, C, O])
+        close(g, orc.conv2d_transpose_kernel_grad(x, dy, s, (kh, kw)), "conv2d_transpose_kernel_grad at batch 64")
         return
     # input gradient: strides, dy dims, filter dims, input dims (:171-193)
     (e, _), (g, _), code = seam.run_both(A, "conv2d_input_grad", [dy, k, None, np.zeros((N, H, W, C), np.float32), None],

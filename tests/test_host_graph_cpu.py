@@ -39,6 +39,25 @@ def test_dcgan_forward_losses_and_all_gradients_vs_torch_f64(cpu_dump):
         np.testing.assert_allclose(got, exp, rtol=2e-4, atol=tol, err_msg=key)
 
 
+def test_labelled_discriminator_pass_vs_torch_f64(tmp_path):
+    """The discriminator alone on labelled images (random 0/1 labels): layers, logits, loss, all dW / db and
+    the gradient of the input images."""
+    import __graft_entry__ as ge
+    path = str(tmp_path / "disc.npz")
+    env = dict(os.environ, RT_MODE="CPU", OMP_NUM_THREADS="8")
+    subprocess.run([sys.executable, os.path.join(ROOT, "tests", "dcgan_reference.py"), "3", "11", path, "disc"],
+                   check=True, env=env, timeout=600)
+    got = dict(np.load(path))
+    w, _, x = dr.synthetic(3, 11, ge.load_package().hostabi.var_shapes())
+    y = dr.labels(3, 11)
+    ref = dr.torch_disc(w, x, y)
+    assert set(ref) == set(got) and len(ref) == 17
+    for key, exp in ref.items():
+        tol = 2e-5 * max(1.0, float(np.abs(exp).max()))
+        np.testing.assert_allclose(got[key].reshape(-1).astype(np.float64), exp, rtol=2e-4, atol=tol, err_msg=key)
+    assert np.abs(ref["grad_disc_loss_x_real"]).max() > 0
+
+
 def test_adam_step_moves_parameters_as_the_closed_form_says(cpu_dump):
     """After the first Adam step (m = (1-b1) g, v = (1-b2) g^2, t = 1) every parameter moves by
     lr * sign(g) / (1 + eps / (sqrt(1-b2) |g|)): |delta| ~= 2e-4 wherever |g| >> 3e-7."""
