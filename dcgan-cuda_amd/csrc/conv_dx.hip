@@ -87,6 +87,17 @@ int conv_dx(const char* who, const float* dy, const float* dy2, const float* k, 
             slabs += t * ((all[q].K + BK - 1) / BK);
         }
         cfg = narrower_if_split(cfg, tiles, slabs);
+        if (g_force_tile_width && cfg.bm == 128 && C > 64) cfg.bn = g_force_tile_width;
+        if (g_tuning_width && cfg.bm == 128 && C > 64) cfg.bn = g_tuning_width;
+        if (width_is_measured(cfg, tiles))
+        {
+            TuneKey key{MODE_DX, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left, pair ? 1 : 0, num_cus()};
+            int width = 128;
+            DH_TRY(measured_width(key, as_stream(stream), [&] {
+                return conv_dx(who, dy, dy2, k, dx, dx2, N, Ho, Wo, O, kh, kw, C, sh, sw, pad_top, pad_left, H, W, bias, act, alpha, stream);
+            }, &width));
+            cfg.bn = width;
+        }
     }
     for (int q = 0; q < n_live; ++q)
         total_tiles_m += (all[q].M + cfg.bm - 1) / cfg.bm;

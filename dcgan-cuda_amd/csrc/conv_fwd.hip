@@ -38,6 +38,17 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     {
         const long tiles = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
         cfg = narrower_if_split(cfg, tiles, tiles * ((p.phase[0].K + BK - 1) / BK));
+        if (g_force_tile_width && cfg.bm == 128 && O > 64) cfg.bn = g_force_tile_width;
+        if (g_tuning_width && cfg.bm == 128 && O > 64) cfg.bn = g_tuning_width;
+        if (width_is_measured(cfg, tiles))
+        {
+            TuneKey key{MODE_FWD, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left, pair ? 1 : 0, num_cus()};
+            int width = 128;
+            DH_TRY(measured_width(key, as_stream(stream), [&] {
+                return conv_fwd(who, x, x2, k, y, y2, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias, act, alpha, stream);
+            }, &width));
+            cfg.bn = width;
+        }
     }
     const long wgs = (long)((p.phase[0].M + cfg.bm - 1) / cfg.bm) * ((O + cfg.bn - 1) / cfg.bn) * instances;
     if (takes_fast_path(veca, vecb))

@@ -34,6 +34,8 @@ int num_cus();
 // Level 1 times the convolution kernels only (a few dozen launches per training iteration, so the
 // events barely disturb it); level 2 also times the reductions, dense and element-wise kernels.
 bool profiling(int level = 1);
+// Launches between prof_pause(true) and prof_pause(false) are not recorded (calls nest).
+void prof_pause(bool on);
 // `issued` (convolution kernels): the FLOPs the matrix cores are issued for the launch, 0 = not known.
 int prof_begin(const char* name, double work, hipStream_t st, int level = 1, double issued = 0.0);
 void prof_end(int handle, hipStream_t st);
@@ -76,6 +78,7 @@ bool dk_thin_takes(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, in
 // Test and tuning switches (dh_debug_force_generic_conv, dh_debug_force_splitk).
 extern bool g_force_generic;  // route every convolution through the general kernel
 extern int g_force_splitk;    // > 0: this many k splits (at most one per k-slab) instead of the automatic choice
+extern int g_force_tile_width;  // 64 / 128: width of the 128-row tiles of wide forward / input-gradient launches
 
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 

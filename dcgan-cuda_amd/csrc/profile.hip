@@ -25,6 +25,7 @@ struct ProfTotal
     double ms, work, issued;
 };
 int g_level = 0;   // 0 off, 1 convolution kernels, 2 every tagged kernel
+int g_paused = 0;  // > 0: launches are not recorded (the library's own measuring runs)
 std::vector<ProfRecord> g_open;      // begun, not yet ended
 std::vector<ProfRecord> g_pending;   // ended, not yet read
 std::vector<hipEvent_t> g_pool;
@@ -55,11 +56,12 @@ hipEvent_t take_event()
 }
 }  // namespace
 
-bool profiling(int level) { return g_level >= level; }
+bool profiling(int level) { return g_paused == 0 && g_level >= level; }
+void prof_pause(bool on) { g_paused += on ? 1 : -1; }
 
 int prof_begin(const char* name, double work, hipStream_t st, int level, double issued)
 {
-    if (g_level < level)
+    if (g_paused > 0 || g_level < level)
         return -1;
     ProfRecord r{};
     r.tag = tag_of(name);

@@ -134,6 +134,7 @@ int workspace(size_t bytes, void** ptr, hipStream_t stream)
 
 bool g_force_generic = false;
 int g_force_splitk = 0;
+int g_force_tile_width = 0;
 
 }  // namespace dh
 
@@ -352,6 +353,14 @@ int dh_debug_force_splitk(int splits)
 {
     if (splits < 0) return fail(DH_EINVAL, "dh_debug_force_splitk: negative split count");
     g_force_splitk = splits;
+    return 0;
+}
+
+int dh_debug_force_tile_width(int width)
+{
+    if (width != 0 && width != 64 && width != 128)
+        return fail(DH_EINVAL, "dh_debug_force_tile_width: width must be 0, 64 or 128");
+    g_force_tile_width = width;
     return 0;
 }
 

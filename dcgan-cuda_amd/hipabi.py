@@ -47,6 +47,7 @@ _SIGS = {
     "dh_pool_stats": [C.POINTER(_sz)] * 4,
     "dh_debug_force_generic_conv": [_i],
     "dh_debug_force_splitk": [_i],
+    "dh_debug_force_tile_width": [_i],
     "dh_profile_enable": [_i],
     "dh_profile_reset": [],
     "dh_profile_read": [C.c_char_p, _sz],

@@ -126,6 +126,12 @@ int dh_debug_force_generic_conv(int on);
  * The partial sums are added in split order by a second kernel, so results are reproducible. */
 int dh_debug_force_splitk(int splits);
 
+/* Test and tuning hook: width 64 or 128 makes every forward / input-gradient launch of the buffer-load
+ * kernel whose result has more than 64 columns use 128 x width tiles; 0 restores the library's choice
+ * (by rule for launches the device holds at once, by measurement for larger ones, see dh_conv2d_fwd).
+ * Without a split the tile width does not change any sum: results are identical to the bit. */
+int dh_debug_force_tile_width(int width);
+
 /* ---- convolutions: fp32 implicit GEMM on MFMA, no im2col buffer ------------------------------ */
 
 /* conv2d forward, optionally with the bias add and activation that follow it fused in.

@@ -376,7 +376,7 @@ def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
 
 @pytest.mark.parametrize("case", [  # (N, H, W, C, kh, kw, O, stride), operator, tile the launch must take
     ((64, 64, 64, 16, 3, 3, 128, 2), "fwd", "128x128"),   # 512 square tiles fill the device unsplit
-    ((64, 64, 64, 128, 3, 3, 16, 2), "dx", "128x128"),    # ... the input gradient's four phases
+    ((64, 64, 64, 128, 3, 3, 16, 2), "dx", "measured"),   # 2048 square tiles, several rounds: the width is timed
     ((64, 32, 32, 16, 3, 3, 256, 2), "fwd", "128x64"),    # 256 square tiles: twice as many narrow ones need no split
     ((64, 8, 8, 64, 5, 5, 256, 2), "fwd", "128x64"),      # a small split launch: narrow tiles, pixels in sorted order
     ((64, 8, 8, 128, 5, 5, 64, 2), "dx", "128x64"),       # ... input gradient
@@ -384,8 +384,10 @@ def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
 ])
 def test_tile_width_follows_the_size_of_the_launch(be, orc, case):
     """Forward and input-gradient launches take 128x64 tiles where 128x128 tiles would need a split
-    that the narrower ones avoid or make cheaper; which tile ran is read from the kernel tags of the
-    profiling interface, the result is checked against the oracle."""
+    that the narrower ones avoid or make cheaper; a launch of more square tiles than the device holds at
+    once takes whichever width the library measured to be faster on its first call (the measuring runs
+    themselves are not recorded).  Which tile ran is read from the kernel tags of the profiling interface,
+    the result is checked against the oracle."""
     import __graft_entry__ as ge
     A = ge.load_package().hipabi
     if A.device_info()["compute_units"] != 256:
@@ -409,8 +411,34 @@ def test_tile_width_follows_the_size_of_the_launch(be, orc, case):
         tags = [r["name"] for r in A.profile_read()]
     finally:
         A.profile_enable(0)
-    assert tags == ["conv_igemm_fast<%s,%s>" % (op, tile)], tags
+    allowed = ("128x128", "128x64") if tile == "measured" else (tile,)
+    assert tags in [["conv_igemm_fast<%s,%s>" % (op, t)] for t in allowed], tags
     close(got, exp, scale=scale, what=op)
+
+
+def test_tile_width_does_not_change_an_unsplit_result(be):
+    """Where the width is chosen by measurement the launch is unsplit with either width, so every output is
+    the same sum in the same order: forward product and input gradient are identical to the bit with 128x128
+    and 128x64 tiles, and so is the library's own choice."""
+    shape = (64, 64, 64, 128, 3, 3, 128, 2)        # 512 x 1 and 4 x 512 square tiles, contraction of 72 slabs
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(43, *shape)
+    results = {}
+    try:
+        for width in (128, 64, 0):
+            print("width", width, flush=True)
+            be.lib.dh_debug_force_tile_width(width)
+            if width:
+                be.lib.dh_debug_force_splitk(1)
+            results[width] = (be.conv2d(x, k, (s, s)), be.conv2d_input_grad(dy, k, s, (H, W)))
+            be.lib.dh_debug_force_splitk(0)
+    finally:
+        be.lib.dh_debug_force_tile_width(0)
+        be.lib.dh_debug_force_splitk(0)
+    for op in (0, 1):
+        np.testing.assert_array_equal(results[64][op], results[128][op])
+    # the input gradient's 2048 tiles are a measured launch: whichever width won, the bits are these
+    np.testing.assert_array_equal(results[0][1], results[128][1])
 
 
 def test_split_with_more_workgroups_than_the_table_holds(be, orc):
