@@ -19,10 +19,28 @@ namespace
 constexpr int TS = 64;   // output tile
 constexpr int KS = 16;   // k slab
 
+// activation applied in the write-out (DH_ACT_NONE: none)
+struct Act
+{
+    int code;
+    float alpha;
+    __device__ __forceinline__ float operator()(float v) const
+    {
+        switch (code)
+        {
+        case DH_ACT_RELU: return v < 0.f ? 0.f : v;
+        case DH_ACT_LEAKY: return v < 0.f ? alpha * v : v;
+        case DH_ACT_TANH: return tanhf(v);
+        case DH_ACT_SIGMOID: return 1.f / (1.f + expf(-v));
+        default: return v;
+        }
+    }
+};
+
 // C[i,j] = sum_k A(i,k) * B(k,j) (+ bias[j]),  A(i,k) = a[i*sai + k*sak],  B(k,j) = b[k*sbk + j*sbj]
 __global__ __launch_bounds__(256) void gemm_tiled(const float* __restrict__ a, const float* __restrict__ b,
                                                   const float* __restrict__ bias, float* __restrict__ out,
-                                                  int M, int K, int P, size_t sai, size_t sak, size_t sbk, size_t sbj)
+                                                  int M, int K, int P, size_t sai, size_t sak, size_t sbk, size_t sbj, Act act)
 {
     __shared__ float la[KS][TS + 1];
     __shared__ float lb[KS][TS + 1];
@@ -66,7 +84,7 @@ __global__ __launch_bounds__(256) void gemm_tiled(const float* __restrict__ a, c
         {
             const int i = i0 + ty + 16 * q, j = j0 + tx + 16 * r;
             if (i < M && j < P)
-                out[(size_t)i * P + j] = acc[q][r] + (bias ? bias[j] : 0.f);
+                out[(size_t)i * P + j] = act(acc[q][r] + (bias ? bias[j] : 0.f));
         }
 }
 
@@ -82,7 +100,7 @@ template <int RPT>
 __global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, const float* __restrict__ b,
                                                    const float* __restrict__ bias, float* __restrict__ out,
                                                    int M, int K, int P, size_t sai, size_t sak, size_t sbk,
-                                                   size_t out_si, size_t out_sj)
+                                                   size_t out_si, size_t out_sj, Act act)
 {
     constexpr int ROWS = 4 * RPT;
     constexpr int LD = ROWS + 4;   // keeps 16-byte alignment of a wavefront's rows
@@ -172,7 +190,7 @@ __global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, 
         {
             const int i = i0 + ty * RPT + r;
             if (i < M)
-                out[(size_t)i * out_si + (size_t)j * out_sj] = acc[r] + bj;
+                out[(size_t)i * out_si + (size_t)j * out_sj] = act(acc[r] + bj);
         }
     }
 }
@@ -183,16 +201,24 @@ __global__ __launch_bounds__(256) void gemm_skinny(const float* __restrict__ a, 
 // flight per lane, and wavefront 0 adds the four partial sums in a fixed order.  (gemm_skinny<1> walks
 // the whole contraction in one wavefront, four loads at a time, while three wavefronts idle: 10 us
 // against 5 for this shape.)
+// With a second pair of operands (a2, b2 non-null) the contraction runs over both, K elements each: the
+// first two wavefronts take the first pair, the other two the second.
 __global__ __launch_bounds__(256) void gemv_rows(const float* __restrict__ a, const float* __restrict__ b,
+                                                 const float* __restrict__ a2, const float* __restrict__ b2,
                                                  const float* __restrict__ bias, float* __restrict__ out, int K, int P,
-                                                 size_t sak, size_t sbk)
+                                                 size_t sak, size_t sbk, Act act)
 {
     __shared__ float part[4][64];
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     const int j = blockIdx.x * 64 + tx;
     const int jc = j < P ? j : P - 1;
-    const int kq = (K + 3) / 4;
-    const int k0 = ty * kq, k1 = K < k0 + kq ? K : k0 + kq;
+    const bool two = a2 != nullptr;
+    const int shares = two ? 2 : 4;          // wavefronts per pair of operands
+    const int kq = (K + shares - 1) / shares;
+    const int share = two ? (ty & 1) : ty;
+    const float* __restrict__ av = two && ty >= 2 ? a2 : a;
+    const float* __restrict__ bm = two && ty >= 2 ? b2 : b;
+    const int k0 = share * kq, k1 = K < k0 + kq ? K : k0 + kq;
     float s = 0.f;
     for (int k = k0; k < k1; k += 16)
     {
@@ -202,8 +228,8 @@ __global__ __launch_bounds__(256) void gemv_rows(const float* __restrict__ a, co
         {
             const bool live = k + u < k1;
             const int kk = live ? k + u : k0;   // a valid row; its product is dropped
-            w[u] = b[(size_t)kk * sbk + jc];
-            x[u] = live ? a[(size_t)kk * sak] : 0.f;
+            w[u] = bm[(size_t)kk * sbk + jc];
+            x[u] = live ? av[(size_t)kk * sak] : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < 16; ++u)
@@ -212,14 +238,14 @@ __global__ __launch_bounds__(256) void gemv_rows(const float* __restrict__ a, co
     part[ty][tx] = s;
     __syncthreads();
     if (ty == 0 && j < P)
-        out[j] = ((part[0][tx] + part[1][tx]) + part[2][tx]) + part[3][tx] + (bias ? bias[j] : 0.f);
+        out[j] = act(((part[0][tx] + part[1][tx]) + part[2][tx]) + part[3][tx] + (bias ? bias[j] : 0.f));
 }
 
 // one workgroup per output element: 256 lanes stride over k, then a fixed LDS tree
 __global__ __launch_bounds__(256) void gemm_block_per_output(const float* __restrict__ a, const float* __restrict__ b,
                                                              const float* __restrict__ bias, float* __restrict__ out,
                                                              int M, int K, int P, size_t sai, size_t sak, size_t sbk,
-                                                             size_t sbj)
+                                                             size_t sbj, Act act)
 {
     __shared__ float lds[256];
     const size_t o = blockIdx.x;
@@ -247,12 +273,12 @@ __global__ __launch_bounds__(256) void gemm_block_per_output(const float* __rest
         if ((int)threadIdx.x < w) lds[threadIdx.x] += lds[threadIdx.x + w];
         __syncthreads();
     }
-    if (threadIdx.x == 0) out[o] = lds[0] + (bias ? bias[j] : 0.f);
+    if (threadIdx.x == 0) out[o] = act(lds[0] + (bias ? bias[j] : 0.f));
     (void)M;
 }
 
 int run_gemm(const char* who, const float* a, const float* b, const float* bias, float* out, size_t m, size_t n,
-             size_t p, size_t sai, size_t sak, size_t sbk, size_t sbj, void* stream)
+             size_t p, size_t sai, size_t sak, size_t sbk, size_t sbj, void* stream, Act act = Act{DH_ACT_NONE, 0.f})
 {
     DH_TRY(ensure_init());
     if (m == 0 || p == 0) return 0;
@@ -264,26 +290,28 @@ int run_gemm(const char* who, const float* a, const float* b, const float* bias,
     {
         // too few workgroups of 64 rows to fill the device: 16 rows each
         hipLaunchKernelGGL(gemm_skinny<4>, dim3((unsigned)((p + 63) / 64), (unsigned)((m + 15) / 16)), dim3(256), 0, st, a, b,
-                           bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+                           bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1, act);
     }
     else if (n <= SK_MAXK && sbj == 1 && p >= 64 && m > 4)
         hipLaunchKernelGGL(gemm_skinny<16>, dim3((unsigned)((p + 63) / 64), (unsigned)((m + 63) / 64)), dim3(256), 0, st, a, b,
-                           bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+                           bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, p, (size_t)1, act);
     else if (n <= SK_MAXK && sbj == 1 && p >= 64 && m == 1)
-        hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((p + 63) / 64)), dim3(256), 0, st, a, b, bias, out, (int)n, (int)p, sak, sbk);
+        hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((p + 63) / 64)), dim3(256), 0, st, a, b, (const float*)nullptr,
+                           (const float*)nullptr, bias, out, (int)n, (int)p, sak, sbk, act);
     else if (n <= SK_MAXK && sbj == 1 && p >= 64)
         hipLaunchKernelGGL(gemm_skinny<1>, dim3((unsigned)((p + 63) / 64), 1u), dim3(256), 0, st, a, b, bias, out, (int)m,
-                           (int)n, (int)p, sai, sak, sbk, p, (size_t)1);
+                           (int)n, (int)p, sai, sak, sbk, p, (size_t)1, act);
     else if (n <= SK_MAXK && p == 1 && sai == 1 && !bias && m >= 64)
         // a single output column: out[i] = sum_k a[k*sak + i] * b[k*sbk] is the row vector b times the
         // matrix a, whose rows are contiguous -- the same kernel with the roles exchanged
-        hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((m + 63) / 64)), dim3(256), 0, st, b, a, bias, out, (int)n, (int)m, sbk, sak);
+        hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((m + 63) / 64)), dim3(256), 0, st, b, a, (const float*)nullptr,
+                           (const float*)nullptr, bias, out, (int)n, (int)m, sbk, sak, act);
     else if (m * p <= 16384 && n >= 512)
         hipLaunchKernelGGL(gemm_block_per_output, dim3((unsigned)(m * p)), dim3(256), 0, st, a, b, bias, out,
-                           (int)m, (int)n, (int)p, sai, sak, sbk, sbj);
+                           (int)m, (int)n, (int)p, sai, sak, sbk, sbj, act);
     else
         hipLaunchKernelGGL(gemm_tiled, dim3((unsigned)((p + TS - 1) / TS), (unsigned)((m + TS - 1) / TS)), dim3(256), 0,
-                           st, a, b, bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, sbj);
+                           st, a, b, bias, out, (int)m, (int)n, (int)p, sai, sak, sbk, sbj, act);
     DH_LAUNCH_CHECK(who);
     return 0;
 }
@@ -297,9 +325,36 @@ int dh_gemm_nn(const float* a, const float* b, const float* bias, float* out, si
     return run_gemm("dh_gemm_nn", a, b, bias, out, m, n, p, n, 1, p, 1, stream);
 }
 
+int dh_gemm_nn_act(const float* a, const float* b, const float* bias, float* out, size_t m, size_t n, size_t p, int act,
+                   float alpha, void* stream)
+{
+    if (act < DH_ACT_NONE || act > DH_ACT_SIGMOID) return fail(DH_EINVAL, "dh_gemm_nn_act: unknown activation %d", act);
+    return run_gemm("dh_gemm_nn_act", a, b, bias, out, m, n, p, n, 1, p, 1, stream, Act{act, alpha});
+}
+
 int dh_gemm_tn(const float* a, const float* b, float* out, size_t m, size_t n, size_t p, void* stream)
 {
     return run_gemm("dh_gemm_tn", a, b, nullptr, out, m, n, p, 1, m, p, 1, stream);
+}
+
+int dh_gemm_tn_pair_supported(size_t m, size_t n, size_t p) { return p == 1 && m >= 64 && n >= 1 && n <= 64 ? 1 : 0; }
+
+int dh_gemm_tn_pair(const float* a1, const float* b1, const float* a2, const float* b2, float* out, size_t m, size_t n,
+                    size_t p, void* stream)
+{
+    DH_TRY(ensure_init());
+    if (!a1 || !b1 || !a2 || !b2 || !out) return fail(DH_EINVAL, "dh_gemm_tn_pair: null tensor");
+    if (!dh_gemm_tn_pair_supported(m, n, p))
+        return fail(DH_ENOTSUP, "dh_gemm_tn_pair: takes a single output column (p == 1) with m >= 64 and n <= 64");
+    if (m > 0x7fffffff) return fail(DH_EINVAL, "dh_gemm_tn_pair: extent too large");
+    hipStream_t st = as_stream(stream);
+    ProfScope prof("dense gemm", 2.0 * m * (2 * n) * p, st);
+    // out[i] = sum_k b1[k] * a1[k*m + i] + sum_k b2[k] * a2[k*m + i]: the row vectors b times the matrices a,
+    // whose rows are contiguous (see run_gemm's single-output-column case)
+    hipLaunchKernelGGL(gemv_rows, dim3((unsigned)((m + 63) / 64)), dim3(256), 0, st, b1, a1, b2, a2, (const float*)nullptr, out,
+                       (int)n, (int)m, (size_t)1, m, Act{DH_ACT_NONE, 0.f});
+    DH_LAUNCH_CHECK("dh_gemm_tn_pair");
+    return 0;
 }
 
 int dh_gemm_nt(const float* a, const float* b, float* out, size_t m, size_t n, size_t p, void* stream)

@@ -514,6 +514,55 @@ __global__ __launch_bounds__(1024) void mean_reduce(const float* __restrict__ a,
     if (threadIdx.x == 0) out[0] = lds[0] / (float)n;
 }
 
+// Sigmoid cross-entropy of one or two logit vectors in ONE launch: the loss (mean_reduce<RedSce>'s sums, tree
+// and division), its gradient (map2<OpSceGrad>'s formula) and, for two, the sum of the two losses -- the
+// values of the separate launches to the bit, where a training step otherwise issues up to five one-workgroup
+// launches of ~4.5 us each (src/gpu/sigmoid.cu:61-111 and the vect_add that joins the discriminator's losses).
+struct SceHead
+{
+    const float* y[2];
+    const float* x[2];
+    float* loss[2];      // may be null
+    float* grad[2];      // may be null
+    float* sum;          // loss[0] + loss[1], or null
+    int count;
+};
+
+__global__ __launch_bounds__(1024) void sce_head_kernel(const SceHead h, size_t n)
+{
+    __shared__ float lds[1024];
+    const RedSce value{};
+    const OpSceGrad slope{1.f / (float)n};
+    float losses[2] = {0.f, 0.f};
+    for (int q = 0; q < h.count; ++q)
+    {
+        const float* __restrict__ y = h.y[q];
+        const float* __restrict__ x = h.x[q];
+        float* __restrict__ grad = h.grad[q];
+        float s = 0.f;
+        for (size_t i = threadIdx.x; i < n; i += 1024)
+        {
+            const float yi = y[i], xi = x[i];
+            s += value(yi, xi);
+            if (grad)
+                grad[i] = slope(yi, xi);
+        }
+        lds[threadIdx.x] = s;
+        __syncthreads();
+        for (int w = 512; w > 0; w >>= 1)
+        {
+            if ((int)threadIdx.x < w) lds[threadIdx.x] += lds[threadIdx.x + w];
+            __syncthreads();
+        }
+        losses[q] = lds[0] / (float)n;
+        __syncthreads();
+        if (threadIdx.x == 0 && h.loss[q])
+            h.loss[q][0] = losses[q];
+    }
+    if (threadIdx.x == 0 && h.sum)
+        h.sum[0] = losses[0] + losses[1];
+}
+
 // rows whose first-maximum column agrees in y and y_hat (strict '>' keeps the lowest index on ties)
 __global__ __launch_bounds__(1024) void argmax_acc_kernel(const float* __restrict__ y, const float* __restrict__ yh,
                                                           float* __restrict__ out, size_t rows, size_t cols)
@@ -831,6 +880,25 @@ int dh_sigmoid_cross_entropy(const float* y, const float* logits, float* out, si
 
 int dh_sigmoid_cross_entropy_grad(const float* y, const float* logits, float* out, size_t n, void* stream)
 { return run_map2("dh_sigmoid_cross_entropy_grad", y, logits, out, n, stream, OpSceGrad{1.f / (float)n}); }
+
+int dh_sigmoid_cross_entropy_head(const float* y1, const float* logits1, float* loss1, float* grad1, const float* y2,
+                                  const float* logits2, float* loss2, float* grad2, float* loss_sum, size_t n, void* stream)
+{
+    DH_TRY(ensure_init());
+    const bool two = y2 || logits2 || loss2 || grad2;
+    if (!y1 || !logits1 || n == 0 || (two && (!y2 || !logits2)))
+        return fail(DH_EINVAL, "dh_sigmoid_cross_entropy_head: null tensor or n == 0");
+    if (loss_sum && !two)
+        return fail(DH_EINVAL, "dh_sigmoid_cross_entropy_head: a sum of losses needs two logit vectors");
+    SceHead h{};
+    h.y[0] = y1; h.x[0] = logits1; h.loss[0] = loss1; h.grad[0] = grad1;
+    h.y[1] = y2; h.x[1] = logits2; h.loss[1] = loss2; h.grad[1] = grad2;
+    h.sum = loss_sum;
+    h.count = two ? 2 : 1;
+    hipLaunchKernelGGL(sce_head_kernel, dim3(1), dim3(1024), 0, as_stream(stream), h, n);
+    DH_LAUNCH_CHECK("dh_sigmoid_cross_entropy_head");
+    return 0;
+}
 
 int dh_mse(const float* y, const float* y_hat, float* out, size_t rows, size_t cols, void* stream)
 {

@@ -48,6 +48,10 @@ _SIGS = {
     "dh_debug_force_generic_conv": [_i],
     "dh_debug_force_splitk": [_i],
     "dh_debug_force_tile_width": [_i],
+    "dh_sigmoid_cross_entropy_head": [_vp] * 9 + [_sz, _vp],
+    "dh_gemm_nn_act": [_vp] * 4 + [_sz] * 3 + [_i, _f, _vp],
+    "dh_gemm_tn_pair": [_vp] * 5 + [_sz] * 3 + [_vp],
+    "dh_gemm_tn_pair_supported": [_sz] * 3,
     "dh_profile_enable": [_i],
     "dh_profile_reset": [],
     "dh_profile_read": [C.c_char_p, _sz],

@@ -7,6 +7,7 @@
 #include "hip_runner.hh"
 
 #include <algorithm>
+#include <array>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -50,14 +51,20 @@ void conv_dx(const ConvGeom& g, const dbl_t* dy, const dbl_t* k, dbl_t* dx, cons
 // A step is either one node run through the table or one fused call standing for several nodes.
 struct Step
 {
-    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM, ADAM_MULTI, CONV_PAIR } kind = NODE;
-    rt::Node* node = nullptr;    // NODE: the node; CONV_EPILOGUE: the conv node; ACT_BIAS_GRAD: the act-grad node
+    enum Kind { NODE, CONV_EPILOGUE, ACT_BIAS_GRAD, ADAM, ADAM_MULTI, CONV_PAIR, DENSE_EPILOGUE, SCE_HEAD } kind = NODE;
+    // NODE: the node; CONV_EPILOGUE: the conv node; ACT_BIAS_GRAD: the act-grad node; DENSE_EPILOGUE: the
+    // mat_mul_add node (act: its activation); SCE_HEAD: the sigmoid_cross_entropy_grad node
+    rt::Node* node = nullptr;
     rt::Node* bias = nullptr;    // CONV_EPILOGUE: the mat_rvect_add node (may be null)
     rt::Node* act = nullptr;     // CONV_EPILOGUE: the activation node (may be null)
     rt::Node* sum = nullptr;     // ACT_BIAS_GRAD: the mat_sum_cols node
     rt::Node* m1 = nullptr;      // ADAM: moment_update, moment_update2; node = adam_update
     rt::Node* m2 = nullptr;
     rt::Node* add = nullptr;     // ADAM: the `add` node that formed the gradient from two contributions (may be null)
+                                 // SCE_HEAD of two towers: the `add` node that joins their losses
+    rt::Node* loss = nullptr;    // SCE_HEAD: the sigmoid_cross_entropy node on the same labels and logits as `node`
+    rt::Node* node2 = nullptr;   // SCE_HEAD of two towers: gradient and loss node of the second
+    rt::Node* loss2 = nullptr;
     const dbl_t* act_ref = nullptr;  // ACT_BIAS_GRAD: tensor the activation gradient reads
     std::vector<Step> group;     // ADAM_MULTI: the ADAM steps issued as one launch; CONV_PAIR: the two convolution steps
     const dbl_t* grad_sum = nullptr;  // ADAM: gradient tensor that already holds the sum of both contributions
@@ -123,10 +130,16 @@ struct Readers
     }
 };
 
+// The nodes a step stands for (null where it has none in that role).
+std::array<rt::Node*, 10> nodes_of(const Step& s)
+{
+    return {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add, s.loss, s.node2, s.loss2};
+}
+
 // Every tensor a step reads or writes.
 void tensors_of(const Step& s, std::unordered_set<const dbl_t*>& out)
 {
-    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+    for (const rt::Node* n : nodes_of(s))
         if (n)
             for (const dbl_t* t : {(const dbl_t*)n->in1, (const dbl_t*)n->in2, (const dbl_t*)n->in3, (const dbl_t*)n->out1})
                 if (t)
@@ -215,7 +228,7 @@ bool written_once(const Plan& plan, const dbl_t* t)
 {
     int writers = 0;
     auto count = [&](const Step& s) {
-        for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+        for (const rt::Node* n : nodes_of(s))
             if (n && (n->out1 == t || n->out2 == t))
                 writers += 1;
     };
@@ -314,7 +327,8 @@ void defer_bias_sums(Plan& plan, const Keep& keep)
 // interleaved layer by layer); every step still runs after the steps that produce its inputs.
 struct ConvCall
 {
-    int kind = -1;            // 0 forward, 1 input gradient / transpose forward, 2 filter gradient
+    int kind = -1;            // 0 forward, 1 input gradient / transpose forward, 2 filter gradient,
+                              // 3 tr(a) * b of a dense layer (g.N, g.H, g.W hold the product's m, n, p)
     ConvGeom g{};
     const dbl_t* a = nullptr;     // gathered activations (x, dy, x)
     const dbl_t* b = nullptr;     // filter (forward, input gradient) or dy (filter gradient)
@@ -339,6 +353,11 @@ bool conv_call_of(const Step& s, ConvCall& c)
     case rt::Node::OP_CONV2D_TRANSPOSE: c.kind = 1; c.g = geom_transpose(n); c.a = n->in1; c.b = n->in2; break;
     case rt::Node::OP_CONV2D_KERNEL_GRAD: c.kind = 2; c.g = geom_kernel_grad(n); c.a = n->in2; c.b = n->in1; break;
     case rt::Node::OP_CONV2D_TRANSPOSE_KERNEL_GRAD: c.kind = 2; c.g = geom_transpose_kernel_grad(n); c.a = n->in1; c.b = n->in2; break;
+    case rt::Node::OP_TMAT_MAT_MUL:
+        if (s.kind != Step::NODE)
+            return false;
+        c.kind = 3; c.g = ConvGeom{}; c.g.N = (int)n->len1; c.g.H = (int)n->len2; c.g.W = (int)n->len3; c.a = n->in1; c.b = n->in2;
+        break;
     default: return false;
     }
     c.out = n->out1;
@@ -358,6 +377,8 @@ bool conv_call_of(const Step& s, ConvCall& c)
 bool pairable(const ConvCall& c)
 {
     const ConvGeom& g = c.g;
+    if (c.kind == 3)
+        return dh_gemm_tn_pair_supported((std::size_t)g.N, (std::size_t)g.H, (std::size_t)g.W) == 1;
     auto aligned = [](const void* q) { return (reinterpret_cast<std::uintptr_t>(q) & 15) == 0; };
     const double in_bytes = 4.0 * g.N * g.H * g.W * g.C, out_bytes = 4.0 * g.N * g.Ho * g.Wo * g.O;
     const double k_bytes = 4.0 * g.kh * g.kw * g.C * g.O, lim = 2147483648.0;
@@ -379,7 +400,7 @@ bool same_call(const ConvCall& x, const ConvCall& y)
                       g.kh == h.kh && g.kw == h.kw && g.sh == h.sh && g.sw == h.sw && g.pt == h.pt && g.pl == h.pl;
     if (!geom || x.kind != y.kind)
         return false;
-    if (x.kind == 2)
+    if (x.kind >= 2)
         return true;
     return x.b == y.b && x.bias == y.bias && x.act == y.act && x.alpha == y.alpha;
 }
@@ -395,7 +416,8 @@ bool writes_in_place(const Step& s)
 
 void outputs_of(const Step& s, std::vector<const dbl_t*>& out)
 {
-    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum})
+    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.loss, s.node2, s.loss2,
+                              s.kind == Step::SCE_HEAD ? s.add : nullptr})
         if (n && n->out1)
             out.push_back(n->out1);
 }
@@ -409,7 +431,7 @@ void inputs_of(const Step& s, std::vector<const dbl_t*>& in)
             in.push_back(t);
     };
     add(s.act_ref);
-    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+    for (const rt::Node* n : nodes_of(s))
         if (n)
         {
             add(n->in1);
@@ -464,7 +486,7 @@ void pair_convolutions(Plan& plan, const Keep& keep)
     // forward and input-gradient products with the same filter and epilogue
     for (int i = 0; i < n; ++i)
     {
-        if (!is_conv[i] || call[i].kind == 2 || partner[i] >= 0)
+        if (!is_conv[i] || call[i].kind >= 2 || partner[i] >= 0)
             continue;
         for (int j = i + 1; j < n; ++j)
             if (is_conv[j] && partner[j] < 0 && same_call(call[i], call[j]) && !reach[j][i])
@@ -483,7 +505,7 @@ void pair_convolutions(Plan& plan, const Keep& keep)
         if (pa == producer.end() || pb == producer.end() || pa->second == pb->second)
             return;
         const int a = pa->second, b = pb->second;
-        if (!is_conv[a] || !is_conv[b] || call[a].kind != 2 || !same_call(call[a], call[b]) || partner[a] >= 0 ||
+        if (!is_conv[a] || !is_conv[b] || call[a].kind < 2 || !same_call(call[a], call[b]) || partner[a] >= 0 ||
             partner[b] >= 0 || call[a].out != adam.add->in1 || call[b].out != adam.add->in2 ||
             reads[adam.add->in1] != 1 || reads[adam.add->in2] != 1 || keep.count(adam.add->in1) || keep.count(adam.add->in2))
             return;
@@ -498,6 +520,26 @@ void pair_convolutions(Plan& plan, const Keep& keep)
         for (Step& g : st[i].group)
             consider(g);
     }
+    // two loss-plus-gradient steps whose losses an `add` joins: one launch for the three (the discriminator's
+    // loss on the real and on the generated batch, dcgan/main.cu:304-307)
+    std::vector<int> joined(n, -1);       // the `add` step of a pair of SCE_HEAD steps (at both members), -1 otherwise
+    for (int k = 0; k < n; ++k)
+    {
+        const Step& add = st[k];
+        if (add.kind != Step::NODE || add.node->type != rt::Node::OP_ADD || add.node->len1 != 1)
+            continue;
+        auto pa = producer.find(add.node->in1), pb = producer.find(add.node->in2);
+        if (pa == producer.end() || pb == producer.end() || pa->second == pb->second)
+            continue;
+        const int a = pa->second, b = pb->second;
+        if (st[a].kind != Step::SCE_HEAD || st[b].kind != Step::SCE_HEAD || st[a].node2 || st[b].node2 ||
+            partner[a] >= 0 || partner[b] >= 0 || st[a].loss->out1 != add.node->in1 || st[b].loss->out1 != add.node->in2 ||
+            st[a].node->len1 != st[b].node->len1)
+            continue;
+        partner[a] = b;
+        partner[b] = a;
+        joined[a] = joined[b] = k;
+    }
     bool any = false;
     for (int i = 0; i < n; ++i)
         any = any || partner[i] >= 0;
@@ -508,6 +550,9 @@ void pair_convolutions(Plan& plan, const Keep& keep)
     std::vector<int> node_of(n);
     for (int i = 0; i < n; ++i)
         node_of[i] = partner[i] >= 0 && partner[i] < i ? partner[i] : i;
+    for (int i = 0; i < n; ++i)
+        if (joined[i] >= 0)
+            node_of[joined[i]] = node_of[i];
     std::vector<std::vector<int>> succ(n);
     std::vector<int> waiting(n, 0);
     for (int i = 0; i < n; ++i)
@@ -545,6 +590,16 @@ void pair_convolutions(Plan& plan, const Keep& keep)
             --waiting[v];
         if (partner[pick] < 0)
             order.push_back(st[pick]);
+        else if (joined[pick] >= 0)
+        {
+            // in the order of the `add` node's operands
+            Step both = st[pick];
+            const Step& other = st[partner[pick]];
+            both.node2 = other.node;
+            both.loss2 = other.loss;
+            both.add = st[joined[pick]].node;
+            order.push_back(both);
+        }
         else
         {
             int first = pick, second = partner[pick];
@@ -593,10 +648,58 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const Keep& keep, bool fuse)
     // ... and the caller does not read it either: t need not exist after the run
     auto only_reader = [&](const dbl_t* t, rt::Node* who) { return !keep.count(t) && sole_reader(t, who); };
 
+    // Whether an activation node may be folded into the launch that produces its input z: z is read only by
+    // that activation and by gradient nodes that can take the activation's OUTPUT instead (same sign for
+    // relu and for leaky with alpha > 0), and the caller does not ask for z itself.
+    auto foldable_activation = [&](const dbl_t* z) -> rt::Node* {
+        if (keep.count(z))
+            return nullptr;
+        rt::Node* act = nullptr;
+        for (rt::Node* r : readers.of(z))
+        {
+            const int code = act_code(r);
+            if (code >= 0 && r->in1 == z && !act)
+                act = r;
+            else if ((r->type == rt::Node::OP_RELU_GRAD || r->type == rt::Node::OP_LEAKY_RELU_GRAD) && r->in1 == z &&
+                     r->in2 != z)
+                ;  // redirected to the activation's output
+            else
+                return nullptr;
+        }
+        if (!act)
+            return nullptr;
+        const int code = act_code(act);
+        for (rt::Node* r : readers.of(z))
+        {
+            if (r == act)
+                continue;
+            if (r->type == rt::Node::OP_RELU_GRAD && code != DH_ACT_RELU)
+                return nullptr;
+            if (r->type == rt::Node::OP_LEAKY_RELU_GRAD && !(code == DH_ACT_LEAKY && act->alpha_leaky > 0.f))
+                return nullptr;
+        }
+        return act;
+    };
+
     for (rt::Node* n : nodes)
     {
         if (absorbed.count(n))
             continue;
+        if (n->type == rt::Node::OP_MAT_MUL_ADD)
+        {
+            // dense layer: mat_mul_add -> activation in the product's write-out
+            rt::Node* act = foldable_activation(n->out1);
+            if (!act || absorbed.count(act))
+                continue;
+            Step s;
+            s.kind = Step::DENSE_EPILOGUE;
+            s.node = n;
+            s.act = act;
+            absorbed.insert(act);
+            z_alias[n->out1] = act->out1;
+            fused_at[act] = s;
+            continue;
+        }
         if (is_conv_like(n))
         {
             // conv -> mat_rvect_add(conv_out, b) [-> activation(z)]
@@ -612,43 +715,12 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const Keep& keep, bool fuse)
             s.bias = bias;
             absorbed.insert(bias);
             rt::Node* last = bias;
-            // The activation may be folded in when z is read only by it and by gradient nodes that
-            // can take the activation's OUTPUT instead (same sign for relu and for leaky with
-            // alpha > 0), and the caller does not ask for z itself.
-            rt::Node* act = nullptr;
-            bool ok = !keep.count(bias->out1);
-            for (rt::Node* r : readers.of(bias->out1))
+            if (rt::Node* act = foldable_activation(bias->out1))
             {
-                const int code = act_code(r);
-                if (code >= 0 && r->in1 == bias->out1 && !act)
-                    act = r;
-                else if ((r->type == rt::Node::OP_RELU_GRAD || r->type == rt::Node::OP_LEAKY_RELU_GRAD) &&
-                         r->in1 == bias->out1 && r->in2 != bias->out1)
-                    ;  // redirected below
-                else
-                    ok = false;
-            }
-            if (ok && act)
-            {
-                const int code = act_code(act);
-                bool sign_safe = true;
-                for (rt::Node* r : readers.of(bias->out1))
-                {
-                    if (r == act)
-                        continue;
-                    if (r->type == rt::Node::OP_RELU_GRAD && code != DH_ACT_RELU)
-                        sign_safe = false;
-                    if (r->type == rt::Node::OP_LEAKY_RELU_GRAD &&
-                        !(code == DH_ACT_LEAKY && act->alpha_leaky > 0.f))
-                        sign_safe = false;
-                }
-                if (sign_safe)
-                {
-                    s.act = act;
-                    absorbed.insert(act);
-                    z_alias[bias->out1] = act->out1;
-                    last = act;
-                }
+                s.act = act;
+                absorbed.insert(act);
+                z_alias[bias->out1] = act->out1;
+                last = act;
             }
             fused_at[last] = s;
         }
@@ -718,6 +790,34 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const Keep& keep, bool fuse)
             }
         }
     }
+    // sigmoid cross-entropy: the loss node and its gradient node on the same labels and logits become one
+    // launch, issued where the first of the two stood (both outputs are still written)
+    for (rt::Node* n : nodes)
+    {
+        if (n->type != rt::Node::OP_SIGMOID_CROSS_ENTROPY_GRAD || absorbed.count(n))
+            continue;
+        rt::Node* loss = nullptr;
+        for (rt::Node* r : readers.of(n->in2))
+            if (r->type == rt::Node::OP_SIGMOID_CROSS_ENTROPY && r->in1 == n->in1 && r->in2 == n->in2 && r->len1 == n->len1 &&
+                !absorbed.count(r))
+                loss = r;
+        if (!loss)
+            continue;
+        Step s;
+        s.kind = Step::SCE_HEAD;
+        s.node = n;
+        s.loss = loss;
+        absorbed.insert(n);
+        absorbed.insert(loss);
+        rt::Node* first = n;
+        for (rt::Node* q : nodes)
+            if (q == n || q == loss)
+            {
+                first = q;
+                break;
+            }
+        fused_at[first] = s;
+    }
     for (rt::Node* n : nodes)
     {
         auto f = fused_at.find(n);
@@ -734,10 +834,10 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const Keep& keep, bool fuse)
         }
         if (absorbed.count(n))
             continue;
-        // a conv whose epilogue was fused is emitted at the position of the epilogue's last node
+        // a product whose epilogue was fused is emitted at the position of the epilogue's last node
         bool conv_deferred = false;
         for (auto& kv : fused_at)
-            if (kv.second.kind == Step::CONV_EPILOGUE && kv.second.node == n)
+            if ((kv.second.kind == Step::CONV_EPILOGUE || kv.second.kind == Step::DENSE_EPILOGUE) && kv.second.node == n)
                 conv_deferred = true;
         if (conv_deferred)
             continue;
@@ -756,7 +856,8 @@ Plan make_plan(const std::vector<rt::Node*>& nodes, const Keep& keep, bool fuse)
     if (std::getenv("DCGAN_HIP_PLAN_DUMP"))
     {
         // the launches a run turns into, for inspection
-        static const char* kinds[] = {"node", "conv+epilogue", "act-grad+bias-grad", "adam", "adam-multi", "conv pair"};
+        static const char* kinds[] = {"node", "conv+epilogue", "act-grad+bias-grad", "adam", "adam-multi", "pair",
+                                      "dense+activation", "loss+gradient"};
         std::fprintf(stderr, "plan of %zu nodes -> %zu steps\n", nodes.size(), plan.steps.size());
         for (const Step& s : plan.steps)
             std::fprintf(stderr, "  %-20s %-32s len %zu\n", kinds[s.kind], op_name(s.node->type),
@@ -830,6 +931,24 @@ void issue(const Step& s)
         }
         return;
     }
+    case Step::DENSE_EPILOGUE:
+    {
+        rt::Node* d = s.node;
+        CK(dh_gemm_nn_act(d->in1, d->in2, d->in3, s.act->out1, d->len1, d->len2, d->len3, act_code(s.act), s.act->alpha_leaky,
+                          g_stream));
+        return;
+    }
+    case Step::SCE_HEAD:
+    {
+        rt::Node* g = s.node;
+        if (s.node2)
+            CK(dh_sigmoid_cross_entropy_head(g->in1, g->in2, s.loss->out1, g->out1, s.node2->in1, s.node2->in2, s.loss2->out1,
+                                             s.node2->out1, s.add ? s.add->out1 : nullptr, g->len1, g_stream));
+        else
+            CK(dh_sigmoid_cross_entropy_head(g->in1, g->in2, s.loss->out1, g->out1, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                             g->len1, g_stream));
+        return;
+    }
     case Step::ACT_BIAS_GRAD:
     {
         rt::Node* g = s.node;
@@ -869,9 +988,11 @@ void issue(const Step& s)
         else if (a.kind == 1)
             CK(dh_conv2d_dx_pair(a.a, b.a, a.b, a.out, b.out, g.N, g.Ho, g.Wo, g.O, g.kh, g.kw, g.C, g.sh, g.sw, g.pt, g.pl,
                                  g.H, g.W, a.bias, a.act, a.alpha, g_stream));
-        else
+        else if (a.kind == 2)
             CK(dh_conv2d_dk_pair(a.a, a.b, b.a, b.b, a.out, g.N, g.H, g.W, g.C, g.Ho, g.Wo, g.O, g.kh, g.kw, g.sh, g.sw,
                                  g.pt, g.pl, g_stream));
+        else
+            CK(dh_gemm_tn_pair(a.a, a.b, b.a, b.b, a.out, (std::size_t)g.N, (std::size_t)g.H, (std::size_t)g.W, g_stream));
         return;
     }
     case Step::ADAM_MULTI:
@@ -992,7 +1113,7 @@ bool node_touches(const rt::Node* n, const Feed& f)
 
 bool step_touches(const Step& s, const Feed& f)
 {
-    for (const rt::Node* n : {s.node, s.bias, s.act, s.sum, s.m1, s.m2, s.add})
+    for (const rt::Node* n : nodes_of(s))
         if (node_touches(n, f))
             return true;
     if (s.act_ref >= f.begin && s.act_ref < f.end)

@@ -29,6 +29,8 @@ void run_async(rt::NodesList& tasks);
 //   conv2d / conv2d_transpose -> mat_rvect_add -> relu|relu_leaky|tanh      (one launch)
 //   relu_grad|leaky_relu_grad|tanh_grad -> mat_sum_cols                      (one pass)
 //   moment_update + moment_update2 + adam_update of one variable            (one pass)
+//   mat_mul_add -> relu|relu_leaky                                          (one launch)
+//   sigmoid_cross_entropy + sigmoid_cross_entropy_grad on the same logits [x 2 + the add of the losses]  (one launch)
 // Intermediate tensors that other instructions or the caller still read are kept up to date.
 // Off by default (DCGAN_HIP_FUSE=1 or set_fusion(true) turns it on).
 void set_fusion(bool on);

@@ -259,6 +259,14 @@ int dh_act_bias_grad_parts(const float* act_ref, const float* dout, float* dz, f
 int dh_sigmoid_cross_entropy(const float* y, const float* logits, float* out, size_t n, void* stream);
 /* out[i] = (sigmoid(x[i]) - y[i]) / n.  Replaces src/gpu/sigmoid.cu:103-111. */
 int dh_sigmoid_cross_entropy_grad(const float* y, const float* logits, float* out, size_t n, void* stream);
+/* Both of the above for one vector of logits, or for two (y2 / logits2 non-null) together with the sum of the
+ * two losses, in ONE launch: loss_k = dh_sigmoid_cross_entropy(y_k, logits_k), grad_k =
+ * dh_sigmoid_cross_entropy_grad(y_k, logits_k), *loss_sum = *loss1 + *loss2 -- the same values to the bit.  Any
+ * of loss1, grad1, loss2, grad2, loss_sum may be NULL.  For a runner that matches the loss node, its gradient
+ * node and the `add` that joins the discriminator's two losses (dcgan/main.cu:304-307; kernels
+ * src/gpu/sigmoid.cu:61-111, src/gpu/sum.cu:207-214): five one-workgroup launches become one. */
+int dh_sigmoid_cross_entropy_head(const float* y1, const float* logits1, float* loss1, float* grad1, const float* y2,
+                                  const float* logits2, float* loss2, float* grad2, float* loss_sum, size_t n, void* stream);
 /* Mean squared error and its gradient 2/n*(y_hat - y), the loss the reference's conv-gradient tests
  * use (tests/test_conv2d_grad.cu:96).  Replace gpu::mse / mse_grad (src/gpu/sum.cu:15-65). */
 int dh_mse(const float* y, const float* y_hat, float* out, size_t rows, size_t cols, void* stream);
@@ -273,8 +281,18 @@ int dh_argmax_acc(const float* y, const float* y_hat, float* out, size_t rows, s
  * (src/gpu/matmul.cu:12-26, :40-56). */
 int dh_gemm_nn(const float* a, const float* b, const float* bias, float* out,
                size_t m, size_t n, size_t p, void* stream);
+/* dh_gemm_nn followed by an activation (DH_ACT_*) in the write-out: mat_mul_add and the relu of a dense layer
+ * (src/api/layers.cu dense_layer: mat_mul_add then the activation op) as one launch. */
+int dh_gemm_nn_act(const float* a, const float* b, const float* bias, float* out, size_t m, size_t n, size_t p,
+                   int act, float alpha, void* stream);
 /* out (m x p) = tr(a) * b, a is (n x m), b is (n x p).  Replaces tmat_mat_mul (src/gpu/matmul.cu:58-71). */
 int dh_gemm_tn(const float* a, const float* b, float* out, size_t m, size_t n, size_t p, void* stream);
+/* out = tr(a1) * b1 + tr(a2) * b2 as ONE contraction over both (the weight gradients of a dense layer that runs
+ * on two batches and whose sum is all the optimiser reads).  Takes the shapes dh_gemm_tn_pair_supported
+ * answers 1 for (a single output column, p == 1, with m >= 64 and n <= 64) and returns DH_ENOTSUP otherwise. */
+int dh_gemm_tn_pair(const float* a1, const float* b1, const float* a2, const float* b2, float* out, size_t m, size_t n,
+                    size_t p, void* stream);
+int dh_gemm_tn_pair_supported(size_t m, size_t n, size_t p);
 /* out (m x p) = a * tr(b), a is (m x n), b is (p x n).  Replaces mat_tmat_mul (src/gpu/matmul.cu:73-86). */
 int dh_gemm_nt(const float* a, const float* b, float* out, size_t m, size_t n, size_t p, void* stream);
 

@@ -85,6 +85,80 @@ def test_losses(be, orc):
     close(be.mse_grad(a, b), orc.mse_grad(a, b))
 
 
+def test_loss_and_gradient_in_one_launch(be, orc):
+    """dh_sigmoid_cross_entropy_head: loss and gradient of one or two logit vectors and the sum of two losses
+    are the values of the separate entry points to the bit."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    lib = A.load()
+    rng = np.random.default_rng(21)
+    for n in (1, 64, 512, 5000):
+        print("n", n, flush=True)
+        xs = [rng.uniform(-6, 6, n).astype(np.float32) for _ in range(2)]
+        ys = [(rng.uniform(0, 1, n) > 0.5).astype(np.float32) for _ in range(2)]
+        sep_loss = [be.sigmoid_cross_entropy(y, x) for y, x in zip(ys, xs)]
+        sep_grad = [be.sigmoid_cross_entropy_grad(y, x) for y, x in zip(ys, xs)]
+        dy, dx = [A.Buf.from_numpy(y) for y in ys], [A.Buf.from_numpy(x) for x in xs]
+        loss, grad, total = [A.Buf((1,)) for _ in range(2)], [A.Buf((n,)) for _ in range(2)], A.Buf((1,))
+        A.check(lib.dh_sigmoid_cross_entropy_head(dy[0].ptr, dx[0].ptr, loss[0].ptr, grad[0].ptr, dy[1].ptr, dx[1].ptr,
+                                                  loss[1].ptr, grad[1].ptr, total.ptr, n, None))
+        for q in range(2):
+            np.testing.assert_array_equal(loss[q].numpy()[0], np.float32(sep_loss[q]))
+            np.testing.assert_array_equal(grad[q].numpy(), sep_grad[q])
+        np.testing.assert_array_equal(total.numpy()[0], np.float32(sep_loss[0]) + np.float32(sep_loss[1]))
+        close(grad[0].numpy(), orc.sigmoid_cross_entropy_grad(ys[0], xs[0]))
+        # one vector, gradient only / loss only
+        g1, l1 = A.Buf((n,)), A.Buf((1,))
+        A.check(lib.dh_sigmoid_cross_entropy_head(dy[1].ptr, dx[1].ptr, None, g1.ptr, None, None, None, None, None, n, None))
+        A.check(lib.dh_sigmoid_cross_entropy_head(dy[1].ptr, dx[1].ptr, l1.ptr, None, None, None, None, None, None, n, None))
+        np.testing.assert_array_equal(g1.numpy(), sep_grad[1])
+        np.testing.assert_array_equal(l1.numpy()[0], np.float32(sep_loss[1]))
+    with pytest.raises(A.HipError, match="two logit vectors"):
+        A.check(lib.dh_sigmoid_cross_entropy_head(dy[0].ptr, dx[0].ptr, loss[0].ptr, None, None, None, None, None, total.ptr,
+                                                  n, None))
+
+
+@pytest.mark.parametrize("m,n,p", [(64, 100, 8192), (64, 8192, 1), (9, 33, 17), (1, 64, 8192), (130, 70, 65)])
+def test_dense_with_activation_in_the_write_out(be, orc, m, n, p):
+    """dh_gemm_nn_act = dh_gemm_nn followed by the activation, to the bit (every kernel the shapes route to)."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    lib = A.load()
+    rng = np.random.default_rng(m * 3 + n + p)
+    x = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    w = (rng.standard_normal((n, p)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(p).astype(np.float32) * 0.1
+    z = be.mat_mul_add(x, w, b)
+    dx, dw, db, out = A.Buf.from_numpy(x), A.Buf.from_numpy(w), A.Buf.from_numpy(b), A.Buf((m, p))
+    for act, alpha, ref in ((A.ACT_RELU, 0.0, np.maximum(z, 0)), (A.ACT_LEAKY, 0.2, be.relu_leaky(z, 0.2)),
+                            (A.ACT_NONE, 0.0, z)):
+        A.check(lib.dh_gemm_nn_act(dx.ptr, dw.ptr, db.ptr, out.ptr, m, n, p, act, alpha, None))
+        np.testing.assert_array_equal(out.numpy(), ref)
+    orc.set_threads(8)
+    close(np.maximum(z, 0), orc.relu(orc.mat_mul_add(x, w, b)))
+
+
+@pytest.mark.parametrize("m,n", [(8192, 64), (64, 64), (1000, 37), (200, 1)])
+def test_two_dense_weight_gradients_as_one_contraction(be, orc, m, n):
+    """dh_gemm_tn_pair: tr(a1) b1 + tr(a2) b2 for a single output column."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    lib = A.load()
+    rng = np.random.default_rng(m + n)
+    a = [rng.uniform(-1, 1, (n, m)).astype(np.float32) for _ in range(2)]
+    g = [rng.uniform(-1, 1, (n, 1)).astype(np.float32) for _ in range(2)]
+    assert lib.dh_gemm_tn_pair_supported(m, n, 1) == 1
+    da, dg, out = [A.Buf.from_numpy(v) for v in a], [A.Buf.from_numpy(v) for v in g], A.Buf((m, 1))
+    A.check(lib.dh_gemm_tn_pair(da[0].ptr, dg[0].ptr, da[1].ptr, dg[1].ptr, out.ptr, m, n, 1, None))
+    exp = orc.add(orc.tmm_mul(a[0], g[0]), orc.tmm_mul(a[1], g[1]))
+    close(out.numpy(), exp, scale=4)
+    exp64 = a[0].astype(np.float64).T @ g[0].astype(np.float64) + a[1].astype(np.float64).T @ g[1].astype(np.float64)
+    assert np.abs(out.numpy() - exp64).max() <= 2 * max(np.abs(exp - exp64).max(), 1e-6)
+    assert lib.dh_gemm_tn_pair_supported(m, n, 2) == 0 and lib.dh_gemm_tn_pair_supported(m, 65, 1) == 0
+    with pytest.raises(A.HipError):
+        A.check(lib.dh_gemm_tn_pair(da[0].ptr, dg[0].ptr, da[1].ptr, dg[1].ptr, out.ptr, m, n, 2, None))
+
+
 def test_argmax_is_exact(be, orc):
     rng = np.random.default_rng(4)
     for rows, cols in ((10, 3), (64, 10), (1500, 7), (3, 1)):
