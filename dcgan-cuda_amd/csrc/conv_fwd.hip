@@ -12,6 +12,14 @@ int conv_fwd(const char* who, const float* x, const float* x2, const float* k, f
     DH_TRY(check_geom(who, N, H, W, C, Ho, Wo, O, kh, kw, sh, sw, pad_top, pad_left));
     const bool pair = x2 != nullptr || y2 != nullptr;
     if (!x || !k || !y || (pair && (!x2 || !y2))) return fail(DH_EINVAL, "%s: null tensor", who);
+    if (pair && !g_force_generic)
+    {
+        // the image layer of two towers: one launch over both batches
+        const int rc = conv_fwd_rows(x, x2, k, y, y2, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias, act, alpha,
+                                     as_stream(stream));
+        if (rc != 1)
+            return rc;
+    }
     if (!pair && !g_force_generic)
     {
         const int rc = conv_fwd_thin(x, k, y, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo, bias, act, alpha,
@@ -79,6 +87,17 @@ int dh_conv2d_fwd(const float* x, const float* k, float* y, int N, int H, int W,
 {
     return conv_fwd("dh_conv2d_fwd", x, nullptr, k, y, nullptr, N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo,
                     bias, act, alpha, stream);
+}
+
+int dh_conv2d_fwd_pair_supported(int N, int H, int W, int C, int kh, int kw, int O, int sh, int sw, int pad_top, int pad_left,
+                                 int Ho, int Wo)
+{
+    if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || O <= 0 || Ho <= 0 || Wo <= 0)
+        return 0;
+    if (fwd_rows_takes(N, H, W, C, kh, kw, O, sh, sw, pad_top, pad_left, Ho, Wo))
+        return 1;
+    const double lim = 2147483648.0;
+    return C % BK == 0 && O % 4 == 0 && 4.0 * N * H * W * C < lim && 4.0 * N * Ho * Wo * O < lim && 4.0 * kh * kw * C * O < lim;
 }
 
 int dh_conv2d_fwd_pair(const float* x1, const float* x2, const float* k, float* y1, float* y2, int N, int H, int W,

@@ -713,6 +713,8 @@ struct FwdRowsParams
     const float* k;
     const float* bias;
     float* y;
+    const float* x2;                    // a second batch of N images with the same filter (images N .. 2N-1 of the
+    float* y2;                          // launch), or null
     float alpha;
     int N, H, W, C, Ho, Wo, O, sh, sw, pt, pl;
     int rows_per_task, tasks_per_image, tasks;
@@ -761,8 +763,12 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
             const int row = e < 15 ? di * 15 + e : (di == 0 ? 75 : 76);
             aq[mt][s] = filt[row * 64 + 16 * mt + l16];
         }
-    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)p.y_bytes, 0x00020000);
+    // (a task's image is the same for the whole wavefront: picking the first or the second batch's descriptor is
+    // scalar work)
+    const __amdgpu_buffer_rsrc_t xr1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr1 = __builtin_amdgcn_make_buffer_rsrc(p.y, 0, (int)p.y_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xr2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.x2 ? p.x2 : p.x), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr2 = __builtin_amdgcn_make_buffer_rsrc(p.y2 ? p.y2 : p.y, 0, (int)p.y_bytes, 0x00020000);
     // chunk t*64 + lane of a task's rows: its row and where it is parked
     int put[FR_LOADS], chunk_row[FR_LOADS];
 #pragma unroll
@@ -783,8 +789,11 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
     const uint32_t row_bytes = (uint32_t)p.W * p.C * 4u;
 
     auto issue = [&](int task, dt_f32x4 (&raw)[FR_LOADS]) {
-        const int b = task / p.tasks_per_image;
-        const int h0 = (task - b * p.tasks_per_image) * p.rows_per_task * p.sh - p.pt;
+        const int bb = task / p.tasks_per_image;
+        const int h0 = (task - bb * p.tasks_per_image) * p.rows_per_task * p.sh - p.pt;
+        const bool second = bb >= p.N;
+        const int b = second ? bb - p.N : bb;
+        const __amdgpu_buffer_rsrc_t xr = second ? xr2 : xr1;
         const uint32_t base = ((uint32_t)b * p.H + (uint32_t)h0) * row_bytes;        // (wraps for h0 < 0; such rows are not loaded)
 #pragma unroll
         for (int t = 0; t < FR_LOADS; ++t)
@@ -819,8 +828,11 @@ __global__ __launch_bounds__(64 * FR_WAVES, 2) void fwd_rows(const FwdRowsParams
         if (!first_task)
             issue(task + stride, raw);
         __builtin_amdgcn_sched_barrier(0);      // (the scheduler would sink the loads to where they are used)
-        const int b = task / p.tasks_per_image;
-        const int i0 = (task - b * p.tasks_per_image) * p.rows_per_task;
+        const int bb = task / p.tasks_per_image;
+        const int i0 = (task - bb * p.tasks_per_image) * p.rows_per_task;
+        const bool second = bb >= p.N;
+        const int b = second ? bb - p.N : bb;
+        const __amdgpu_buffer_rsrc_t yr = second ? yr2 : yr1;
 #pragma unroll
         for (int ii = 0; ii < 4; ++ii)
         {
@@ -1192,40 +1204,53 @@ __global__ __launch_bounds__(64 * CT_WAVES, 2) void dx_col2im(const Col2imParams
 namespace dh
 {
 
-// Returns 1 when the shape is not one fwd_rows takes (see the kernel's header), 0 after a launch.
-int conv_fwd_rows(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
-                  int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st)
+// Whether the geometry is one fwd_rows takes (see the kernel's header; the tensors must be 16-byte aligned besides).
+bool fwd_rows_takes(int N, int H, int W, int C, int kh, int kw, int O, int sh, int sw, int pt, int pl, int Ho, int Wo)
 {
     const double x_bytes = (double)N * H * W * C * 4.0, y_bytes = (double)N * Ho * Wo * O * 4.0;
-    if (kh != 5 || kw * C != 15 || O > 64 || O % 16 != 0 || Wo > 32 || sh < 1 || sh > 2 || sw < 1 || sw > 2 || pt < 0 ||
-        pl < 0 || pl * C > FR_LEFT || (W * C) % 4 != 0 || W * C > FR_RS - FR_LEFT - 8 ||
-        FR_LEFT + (31 * sw - pl) * C + 16 > FR_RS || act < DH_ACT_NONE || act > DH_ACT_SIGMOID ||
-        x_bytes >= 4294967040.0 || y_bytes >= 4294967040.0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0 ||
-        (reinterpret_cast<uintptr_t>(y) & 15) != 0)
+    const int rows = 4;   // (the launcher may take fewer rows per task; four must fit)
+    return !(kh != 5 || kw * C != 15 || O > 64 || O % 16 != 0 || Wo > 32 || sh < 1 || sh > 2 || sw < 1 || sw > 2 || pt < 0 ||
+             pl < 0 || pl * C > FR_LEFT || (W * C) % 4 != 0 || W * C > FR_RS - FR_LEFT - 8 ||
+             FR_LEFT + (31 * sw - pl) * C + 16 > FR_RS || x_bytes >= 4294967040.0 || y_bytes >= 4294967040.0 ||
+             (rows - 1) * sh + 5 > FR_STAGED || ((rows - 1) * sh + 5) * (W * C / 4) > FR_LOADS * 64 ||
+             2L * N * ((Ho + rows - 1) / rows) > 0x3fffffffL);
+}
+
+// Returns 1 when the shape is not one fwd_rows takes, 0 after a launch.  x2 / y2 (both null, or both set): a
+// second batch of N images through the same filter in the same launch.
+int conv_fwd_rows(const float* x, const float* x2, const float* k, float* y, float* y2, int N, int H, int W, int C, int kh,
+                  int kw, int O, int sh, int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha,
+                  hipStream_t st)
+{
+    const double x_bytes = (double)N * H * W * C * 4.0, y_bytes = (double)N * Ho * Wo * O * 4.0;
+    const int images = x2 ? 2 * N : N;
+    if (!fwd_rows_takes(N, H, W, C, kh, kw, O, sh, sw, pt, pl, Ho, Wo) || act < DH_ACT_NONE || act > DH_ACT_SIGMOID ||
+        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(x2) |
+          reinterpret_cast<uintptr_t>(y2)) & 15) != 0)
         return 1;
     FwdRowsParams p{};
-    p.x = x; p.k = k; p.bias = bias; p.y = y; p.alpha = alpha;
+    p.x = x; p.k = k; p.bias = bias; p.y = y; p.x2 = x2; p.y2 = y2; p.alpha = alpha;
     p.N = N; p.H = H; p.W = W; p.C = C; p.Ho = Ho; p.Wo = Wo; p.O = O; p.sh = sh; p.sw = sw; p.pt = pt; p.pl = pl;
     p.x_bytes = (uint32_t)x_bytes; p.y_bytes = (uint32_t)y_bytes;
     p.chunks_per_row = W * C / 4;
     // output rows per task: four (they share input rows) when that still gives every wavefront slot a task
     const long slots = (long)num_cus() * FR_WAVES;
     int rows = 4;
-    while (rows > 1 && (long)N * ((Ho + rows - 1) / rows) < slots)
+    while (rows > 1 && (long)images * ((Ho + rows - 1) / rows) < slots)
         rows /= 2;
     p.rows_per_task = rows;
     p.staged = (rows - 1) * sh + 5;
     if (p.staged > FR_STAGED || p.staged * p.chunks_per_row > FR_LOADS * 64)
         return 1;
     p.tasks_per_image = (Ho + rows - 1) / rows;
-    const long tasks = (long)N * p.tasks_per_image;
+    const long tasks = (long)images * p.tasks_per_image;
     if (tasks > 0x3fffffffL)
         return 1;
     p.tasks = (int)tasks;
     long wgs = (tasks + FR_WAVES - 1) / FR_WAVES;
     if (wgs > num_cus())
         wgs = num_cus();
-    const int prof = prof_begin("fwd_rows", 2.0 * N * Ho * Wo * O * kh * kw * C, st, 1, (double)N * Ho * 160.0 * 2048.0);
+    const int prof = prof_begin("fwd_rows", 2.0 * images * Ho * Wo * O * kh * kw * C, st, 1, (double)images * Ho * 160.0 * 2048.0);
     const dim3 grid((unsigned)wgs), block(64 * FR_WAVES);
     switch (act)
     {
@@ -1250,7 +1275,7 @@ int conv_fwd_rows(const float* x, const float* k, float* y, int N, int H, int W,
 int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
                   int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st)
 {
-    if (conv_fwd_rows(x, k, y, N, H, W, C, kh, kw, O, sh, sw, pt, pl, Ho, Wo, bias, act, alpha, st) == 0)
+    if (conv_fwd_rows(x, nullptr, k, y, nullptr, N, H, W, C, kh, kw, O, sh, sw, pt, pl, Ho, Wo, bias, act, alpha, st) == 0)
         return 0;
     const long K = (long)kh * kw * C;
     const size_t x_bytes = (size_t)N * H * W * C * 4;

@@ -66,6 +66,13 @@ int conv_dx_col2im(const float* dy, const float* k, float* dx, int N, int Ho, in
 int conv_fwd_thin(const float* x, const float* k, float* y, int N, int H, int W, int C, int kh, int kw, int O, int sh,
                   int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha, hipStream_t st);
 
+// The image layer's forward product (5 filter rows of 15 values, at most 64 output channels) for two batches of N
+// images that share the filter, in one launch; same return convention.  fwd_rows_takes answers for the geometry.
+int conv_fwd_rows(const float* x, const float* x2, const float* k, float* y, float* y2, int N, int H, int W, int C, int kh,
+                  int kw, int O, int sh, int sw, int pt, int pl, int Ho, int Wo, const float* bias, int act, float alpha,
+                  hipStream_t st);
+bool fwd_rows_takes(int N, int H, int W, int C, int kh, int kw, int O, int sh, int sw, int pt, int pl, int Ho, int Wo);
+
 // Filter gradient of a thin input (at most 80 filter elements per output channel, at most 64 output
 // channels): writes *splits slices of partial sums to the scratch arena and returns them in *part for
 // the caller to add up; same return convention.

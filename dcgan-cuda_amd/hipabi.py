@@ -62,6 +62,7 @@ _SIGS = {
     "dh_conv2d_dx_pair": [_vp] * 5 + [_i] * 13 + [_vp, _i, _f, _vp],
     "dh_conv2d_dk_pair": [_vp] * 5 + [_i] * 13 + [_vp],
     "dh_conv2d_dk_pair_supported": [_i] * 11,
+    "dh_conv2d_fwd_pair_supported": [_i] * 13,
     "dh_bias_add": [_vp, _vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad": [_vp, _vp, _sz, _sz, _vp],
     "dh_bias_grad_parts": [_vp, _vp, _sz, _sz, _vp],

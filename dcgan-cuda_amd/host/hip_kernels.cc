@@ -386,7 +386,10 @@ bool pairable(const ConvCall& c)
     const bool tapwise = c.kind == 0 ? g.C % 16 == 0 : c.kind == 1 ? g.O % 16 == 0 : true;
     const bool sizes_ok = in_bytes < lim && out_bytes < lim && k_bytes < lim && aligned(c.a) && aligned(c.b) &&
                           aligned(c.out) && aligned(c.bias);
-    // the filter gradient of a thin input (the image layer) has a paired kernel of its own
+    // the forward product from a thin input (the image layer) and its filter gradient have paired kernels of their own
+    if (c.kind == 0 && sizes_ok && g.C % 16 != 0 &&
+        dh_conv2d_fwd_pair_supported(g.N, g.H, g.W, g.C, g.kh, g.kw, g.O, g.sh, g.sw, g.pt, g.pl, g.Ho, g.Wo) == 1)
+        return true;
     if (c.kind == 2 && sizes_ok &&
         dh_conv2d_dk_pair_supported(g.N, g.H, g.W, g.C, g.Ho, g.Wo, g.O, g.kh, g.kw, g.sh, g.sw) == 1)
         return true;

@@ -195,6 +195,11 @@ int dh_conv2d_dk_pair(const float* x1, const float* dy1, const float* x2, const 
                       int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw, int pad_top, int pad_left,
                       void* stream);
 int dh_conv2d_dk_pair_supported(int N, int H, int W, int C, int Ho, int Wo, int O, int kh, int kw, int sh, int sw);
+/* 1 when dh_conv2d_fwd_pair has a kernel for the geometry (16-byte aligned tensors assumed): input channels
+ * divisible by 16 and output channels by 4 with every tensor below 2 GiB, or the image layer's shape (a 5-row
+ * filter of 15 values per row, at most 64 output channels, rows of at most 32 output pixels). */
+int dh_conv2d_fwd_pair_supported(int N, int H, int W, int C, int kh, int kw, int O, int sh, int sw, int pad_top,
+                                 int pad_left, int Ho, int Wo);
 
 /* ---- bias and activations: coalesced, vectorised, one pass over HBM ----------------------------- */
 

@@ -672,3 +672,36 @@ def test_paired_filter_gradient_of_a_thin_input(be, orc, shape):
     close(got, exp.astype(np.float32), scale=max(1.0, float(np.abs(exp).max())), what="paired thin filter gradient")
     again = be.conv2d_kernel_grad_pair(dy1, x1, dy2, x2, s, pads)
     np.testing.assert_array_equal(got, again)
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 64, 3, 5, 5, 64, 2), (64, 64, 64, 3, 5, 5, 64, 2), (5, 60, 64, 3, 5, 5, 16, 2)])
+def test_paired_forward_product_of_the_image_layer(be, orc, shape):
+    """conv(x1, k) and conv(x2, k) of the image layer as one launch of the row-wise kernel (the second batch
+    are images N .. 2N-1 of its tasks): each result is the single launch's to the bit, with and without the
+    fused epilogue; the capability query says so beforehand."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    print("shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x1, k, _ = rand_conv_inputs(61, *shape)
+    x2, _, _ = rand_conv_inputs(62, *shape)
+    bias = np.linspace(-0.5, 0.5, O).astype(np.float32)
+    (ph, Ho), (pw, Wo) = same_pad(H, kh, s), same_pad(W, kw, s)
+    assert be.lib.dh_conv2d_fwd_pair_supported(N, H, W, C, kh, kw, O, s, s, ph // 2, pw // 2, Ho, Wo) == 1
+    assert be.lib.dh_conv2d_fwd_pair_supported(2, 8, 8, 3, 5, 5, 6, 2, 2, 1, 1, 4, 4) == 0
+    A.profile_enable(1)
+    A.profile_reset()
+    try:
+        y1, y2 = be.conv2d_pair(x1, x2, k, (s, s))
+        tags = [r["name"] for r in A.profile_read()]
+    finally:
+        A.profile_enable(0)
+    assert tags == ["fwd_rows"], tags
+    np.testing.assert_array_equal(y1, be.conv2d(x1, k, (s, s)))
+    np.testing.assert_array_equal(y2, be.conv2d(x2, k, (s, s)))
+    y1, y2 = be.conv2d_pair(x1, x2, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2)
+    np.testing.assert_array_equal(y1, be.conv2d(x1, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2))
+    np.testing.assert_array_equal(y2, be.conv2d(x2, k, (s, s), bias=bias, act=A.ACT_LEAKY, alpha=0.2))
+    if N <= 5:
+        orc.set_threads(8)
+        close(y2, orc.relu_leaky(orc.bias_add(orc.conv2d(x2, k, (s, s)), bias), 0.2), what="second batch")
