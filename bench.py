@@ -538,6 +538,8 @@ def main():
     ap.add_argument("--profile-every", type=int, default=10,
                     help="bracket the convolution launches with HIP events in every n-th timed iteration")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-drop-in", action="store_true",
+                    help="skip the two extra passes that time the table runner and the list-only plan (profiling runs)")
     ap.add_argument("--host-inputs", action="store_true",
                     help="copy z and the image batch from host memory in every iteration (the PCIe-inclusive "
                          "rate; the default keeps them resident)")
@@ -642,12 +644,14 @@ def main():
         model.sync()
         return ref_steps / (time.perf_counter() - t)
 
-    table_rate = rate(lambda: model.set_fusion(False))
-    table_launches = model.last_launch_count()
-    list_only_rate = rate(lambda: (model.set_fusion(True), model.set_name_results(False)))
-    list_only_launches = model.last_launch_count()
-    model.set_name_results(True)
-    model.set_fusion(bool(args.fusion))
+    table_rate = list_only_rate = table_launches = list_only_launches = None
+    if not args.no_drop_in:
+        table_rate = rate(lambda: model.set_fusion(False))
+        table_launches = model.last_launch_count()
+        list_only_rate = rate(lambda: (model.set_fusion(True), model.set_name_results(False)))
+        list_only_launches = model.last_launch_count()
+        model.set_name_results(True)
+        model.set_fusion(bool(args.fusion))
 
     calibration_copy(A)
 
@@ -709,8 +713,8 @@ def main():
                            "ms_per_step": round(ref_wall * 1e3 / ref_steps, 4),
                            "what": "the reference's own training loop (dcgan/main.cu:378-397): z and the image batch fed "
                                    "from pageable host memory and both losses read back in every iteration"},
-        "table_runner_value": round(table_rate, 3),
-        "drop_in": {
+        "table_runner_value": round(table_rate, 3) if table_rate else None,
+        "drop_in": None if args.no_drop_in else {
             "unit": "iterations/s", "steps": ref_steps,
             "table_runner": {"value": round(table_rate, 3), "launches_in_g_step": table_launches,
                              "what": "every instruction through hip::kernels_list[node->type], in list order, one "

@@ -682,9 +682,23 @@ struct AdamBatch
 // order as the bias gradient's second stage, whose place this takes.  Valid in lane 0.
 __device__ __forceinline__ float sum_of_parts(const float* __restrict__ g, unsigned parts, size_t n, size_t e, unsigned lane)
 {
+    // (sixteen loads are issued before the first add: the parts of a gradient that was written many launches ago
+    // come from HBM, and one round trip per add made a 1024-part sum the longest thing in the optimiser launch;
+    // a missing part adds +0, which leaves the running sum's bits alone)
     float s = 0.f;
-    for (unsigned q = lane; q < parts; q += 64)
-        s += g[(size_t)q * n + e];
+    for (unsigned q0 = lane; q0 < parts; q0 += 64 * 16)
+    {
+        float val[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+        {
+            const unsigned q = q0 + 64u * (unsigned)u;
+            val[u] = q < parts ? g[(size_t)q * n + e] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            s += val[u];
+    }
     for (int off = 32; off > 0; off >>= 1)
         s += __shfl_down(s, off, 64);
     return s;
