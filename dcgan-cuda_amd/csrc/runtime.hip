@@ -38,6 +38,25 @@ struct DeviceState
 std::mutex g_mu;
 DeviceState g_dev[16];
 int g_cur = -1;
+
+// Copies `bytes` (a multiple of 4) from pinned host memory, which the device reads across the bus, to device
+// memory: for the small inputs of a run an ordinary kernel in the launch stream starts sooner than a copy
+// command does.
+__global__ __launch_bounds__(256) void copy_from_pinned(void* __restrict__ dst, const void* __restrict__ src, size_t bytes,
+                                                        bool vec)
+{
+    const size_t stride = (size_t)gridDim.x * 256, tid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    size_t done = 0;
+    if (vec)
+    {
+        const size_t n16 = bytes / 16;
+        for (size_t i = tid; i < n16; i += stride)
+            static_cast<float4*>(dst)[i] = static_cast<const float4*>(src)[i];
+        done = n16 * 16;
+    }
+    for (size_t i = done / 4 + tid; i < bytes / 4; i += stride)
+        static_cast<float*>(dst)[i] = static_cast<const float*>(src)[i];
+}
 }  // namespace
 
 int fail(int code, const char* fmt, ...)
@@ -225,7 +244,21 @@ int dh_memcpy_h2d_staged(void* dst, const void* src, size_t bytes, void* stream)
         slot.bytes = want;
     }
     memcpy(slot.host, src, bytes);
-    DH_HIP(hipMemcpyAsync(dst, slot.host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    // From the staging buffer to the device with a kernel that reads the pinned memory across the bus: in the
+    // launch stream a copy command costs ~20 us before the kernel behind it starts, whatever its size (measured
+    // on the 25 KB latent batch of a training step: 43 us per iteration for two such copies, 11 us for two of
+    // these launches); for megabytes the two are equally fast (the 3 MB image batch: 80 us either way).
+    if (bytes % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 3) == 0)
+    {
+        const bool vec = (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+        size_t blocks = (bytes / 16 + 255) / 256;
+        if (blocks < 1) blocks = 1;
+        if (blocks > 1024) blocks = 1024;
+        hipLaunchKernelGGL(copy_from_pinned, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), dst, slot.host, bytes, vec);
+        DH_LAUNCH_CHECK("copy_from_pinned");
+    }
+    else
+        DH_HIP(hipMemcpyAsync(dst, slot.host, bytes, hipMemcpyHostToDevice, as_stream(stream)));
     DH_HIP(hipEventRecord(slot.done, as_stream(stream)));
     slot.in_flight = true;
     return 0;

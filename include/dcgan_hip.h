@@ -58,10 +58,11 @@ int dh_free(void* ptr);
 int dh_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes);
 /* The same for the inputs a training loop feeds before every run (src/ops/graph.cu:139-147 writes each
  * fed input with tensor_write): the host buffer is copied into a pinned staging buffer of the library
- * (16 of them, used in turn) and from there to the device in `stream` order, so src_host may be
- * reused on return and kernels queued on `stream` afterwards see the data -- but the call does not
- * wait for the work queued before it, as the blocking copy does.  Copies above 64 MiB wait for
- * `stream` and are then blocking. */
+ * (16 of them, used in turn) and from there to the device in `stream` order (by a kernel that reads the
+ * pinned buffer across the bus: it starts sooner than a copy command), so src_host may be reused on
+ * return and kernels queued on `stream` afterwards see the data -- but the call does not wait for the
+ * work queued before it, as the blocking copy does.  Copies above 64 MiB wait for `stream` and are then
+ * blocking. */
 int dh_memcpy_h2d_staged(void* dst_device, const void* src_host, size_t bytes, void* stream);
 int dh_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes);
 int dh_memcpy_d2d(void* dst_device, const void* src_device, size_t bytes, void* stream);
