@@ -343,6 +343,20 @@ def test_taps_in_the_padding_are_skipped(be, orc, shape, splits):
     """Shapes on which the buffer-load kernel leaves out the k-slabs whose taps fall into the
     padding (channel and image counts divisible by 16): forward, input gradient and filter gradient,
     single and paired, automatic split and a forced one, against the oracle."""
+    padding_skip_case(be, orc, shape, splits)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_seeded_random_geometries_with_skipped_taps(be, orc, seed):
+    """The same checks on drawn geometries of that family (image counts 16 ... 80, small odd extents)."""
+    rng = np.random.default_rng(7000 + seed)
+    kh, kw = int(rng.integers(2, 6)), int(rng.integers(2, 6))
+    shape = (16 * int(rng.integers(1, 6)), int(rng.integers(1, 11)), int(rng.integers(1, 11)), 16 * int(rng.integers(1, 4)),
+             kh, kw, 16 * int(rng.integers(1, 6)), int(rng.integers(1, 3)))
+    padding_skip_case(be, orc, shape, int(rng.integers(0, 7)))
+
+
+def padding_skip_case(be, orc, shape, splits):
     import __graft_entry__ as ge
     A = ge.load_package().hipabi
     print("shape", shape, "splits", splits, flush=True)
@@ -705,3 +719,83 @@ def test_paired_forward_product_of_the_image_layer(be, orc, shape):
     if N <= 5:
         orc.set_threads(8)
         close(y2, orc.relu_leaky(orc.bias_add(orc.conv2d(x2, k, (s, s)), bias), 0.2), what="second batch")
+
+
+def seeded_geometry(seed):
+    """A geometry drawn from one of four families: any small shape (general kernel), channels in
+    multiples of 16 / 4 (the vector-load kernels, partial tiles, often split), a thin input (at most
+    4 channels) and a thin result (at most 4 output channels)."""
+    rng = np.random.default_rng(1000 + seed)
+    family = seed % 4
+    kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    # (a stride larger than the filter can leave the last input pixels outside every window: the reference's
+    # unsigned pad arithmetic wraps there, src/gpu/conv2d.cu:88-91, so such geometries have no defined result)
+    s = int(rng.integers(1, min(kh, kw, 3) + 1))
+    N = int(rng.integers(1, 7))
+    H, W = int(rng.integers(3, 21)), int(rng.integers(3, 21))
+    if family == 0:
+        C, O = int(rng.integers(1, 41)), int(rng.integers(1, 41))
+    elif family == 1:
+        C, O = 16 * int(rng.integers(1, 9)), 4 * int(rng.integers(1, 41))
+    elif family == 2:
+        C, O = int(rng.integers(1, 5)), 4 * int(rng.integers(1, 17))
+        H, W = int(rng.integers(8, 41)), int(rng.integers(8, 41))
+    else:
+        C, O = 16 * int(rng.integers(1, 5)), int(rng.integers(1, 5))
+        H, W = int(rng.integers(8, 33)), int(rng.integers(8, 33))
+    return (N, H, W, C, kh, kw, O, s)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_seeded_random_geometries(be, orc, seed):
+    """Forward, input gradient and filter gradient of a drawn geometry, with the automatic split and
+    with a drawn forced one, against the oracle."""
+    import __graft_entry__ as ge
+    A = ge.load_package().hipabi
+    lib = A.load()
+    shape = seeded_geometry(seed)
+    print("seed", seed, "shape", shape, flush=True)
+    N, H, W, C, kh, kw, O, s = shape
+    x, k, dy = rand_conv_inputs(seed, *shape)
+    pads = (same_pad(H, kh, s)[0], same_pad(W, kw, s)[0])
+    orc.set_threads(8)
+    exp_y = orc.conv2d(x, k, (s, s))
+    exp_dx = orc.conv2d_input_grad(dy, k, s, (H, W))
+    exp_dk = orc.conv2d_kernel_grad(dy, x, s, pads)
+    forced = int(np.random.default_rng(seed).integers(2, 7))
+    for splits in (0, forced):
+        A.check(lib.dh_debug_force_splitk(splits))
+        try:
+            close(be.conv2d(x, k, (s, s)), exp_y, what="fwd, splits %d" % splits)
+            close(be.conv2d_input_grad(dy, k, s, (H, W)), exp_dx, what="dx, splits %d" % splits)
+            close(be.conv2d_kernel_grad(dy, x, s, pads), exp_dk, scale=max(1.0, float(np.abs(exp_dk).max())),
+                  what="dk, splits %d" % splits)
+        finally:
+            A.check(lib.dh_debug_force_splitk(0))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_random_transposed_geometries(be, orc, seed):
+    """conv2d_transpose and its two gradients on drawn geometries (x [N,Hi,Wi,Ci] -> [N,s*Hi,s*Wi,Co],
+    filter [kh,kw,Co,Ci]): any small shape, channel counts in multiples of 16 / 4, and the image end
+    (at most 4 output channels)."""
+    rng = np.random.default_rng(5000 + seed)
+    kh, kw = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    s = int(rng.integers(1, min(kh, kw, 3) + 1))
+    N, Hi, Wi = int(rng.integers(1, 6)), int(rng.integers(2, 13)), int(rng.integers(2, 13))
+    family = seed % 3
+    if family == 0:
+        Ci, Co = int(rng.integers(1, 33)), int(rng.integers(1, 33))
+    elif family == 1:
+        Ci, Co = 16 * int(rng.integers(1, 9)), 4 * int(rng.integers(1, 33))
+    else:
+        Ci, Co = 16 * int(rng.integers(1, 5)), int(rng.integers(1, 5))
+    print("seed", seed, "shape", (N, Hi, Wi, Ci, kh, kw, Co, s), flush=True)
+    x = rng.uniform(-1, 1, (N, Hi, Wi, Ci)).astype(np.float32)
+    k = (rng.standard_normal((kh, kw, Co, Ci)) * 0.1).astype(np.float32)
+    dy = rng.uniform(-1, 1, (N, Hi * s, Wi * s, Co)).astype(np.float32)
+    orc.set_threads(8)
+    close(be.conv2d_transpose(x, k, (Hi * s, Wi * s), s), orc.conv2d_transpose(x, k, (Hi * s, Wi * s), s), what="transpose")
+    close(be.conv2d_transpose_input_grad(dy, k, s, (Hi, Wi)), orc.conv2d_transpose_input_grad(dy, k, s, (Hi, Wi)), what="dx")
+    exp = orc.conv2d_transpose_kernel_grad(dy, x, s, (kh, kw))
+    close(be.conv2d_transpose_kernel_grad(dy, x, s, (kh, kw)), exp, scale=max(1.0, float(np.abs(exp).max())), what="dk")
