@@ -12,8 +12,8 @@ time and were never stored.  This script therefore
     ``torch.nn.functional.conv2d`` / ``conv_transpose2d`` and torch autograd for the
     convolutions, numpy closed forms for everything else.
 
-Three expected vectors are additionally asserted against the values written down in the survey
-of the reference (conv2d, conv2d_padding, conv2d_transpose).
+Three expected vectors (conv2d, conv2d_padding, conv2d_transpose) are additionally asserted against
+integer values for the same inputs that were known before this script existed (the literal lists below).
 
 Run once in a container that has the reference mounted:  python tests/golden/make_golden.py
 The JSON it writes is committed; the tests never need the reference tree.
